@@ -187,20 +187,31 @@ class TorchOps:
     def attention_prepare(self, proj, q_off, k_off, v_off, positions, write_slots, plane, n_heads, n_kv_heads, key_dim,
                           value_dim, page_size, q_gain=None, k_gain=None, q_factor=None, freqs=None, rot_dims=0, eps=0.0,
                           write_cache=True, value_norm=True, q_bias=None, k_bias=None, v_bias=None, temp_coef=0.0,
-                          temp_every=1):
+                          temp_every=1, whole_norm=False, pair_half=False):
         n = proj.shape[0]
         H, G, kd, vd = n_heads, n_kv_heads, key_dim, value_dim
 
         def normed(x, gain):
-            return x if gain is None else x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain
+            if gain is None:
+                return x
+            if whole_norm and torch.is_tensor(gain):      # over all heads of the row at once
+                flat = x.reshape(n, -1)
+                return (flat / torch.sqrt((flat * flat).mean(-1, keepdim=True) + eps) * gain).reshape(x.shape)
+            return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain
 
         def turned(x):
             if not rot_dims:
                 return x
             ang = positions.float()[:, None] * freqs[None, :]
             c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
-            a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
             y = x.clone()
+            if pair_half:
+                half = rot_dims // 2
+                a, b = x[..., :half], x[..., half:rot_dims]
+                y[..., :half] = a * c - b * s
+                y[..., half:rot_dims] = b * c + a * s
+                return y
+            a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
             y[..., 0:rot_dims:2] = a * c - b * s
             y[..., 1:rot_dims:2] = b * c + a * s
             return y
@@ -259,7 +270,7 @@ class TorchOps:
         return q.view(n, H * (C + R)), q_plain
 
     def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
-                           scale=None, sink=False, gate=None):
+                           scale=None, sink=False, gate=None, chunk=0):
         n = q.shape[0]
         H, G, kd, vd = n_heads, n_kv_heads, key_dim, value_dim
         scale = scale if scale is not None else kd ** -0.5
@@ -271,7 +282,10 @@ class TorchOps:
         pos, seq = batch.positions.tolist(), batch.row_seq.tolist()
         for r in range(n):
             p = pos[r]
-            js = torch.arange(max(0, p - window + 1) if window > 0 else 0, p + 1)
+            first = max(0, p - window + 1) if window > 0 else 0
+            if chunk > 0:
+                first = max(first, p - p % chunk)
+            js = torch.arange(first, p + 1)
             pg = tables[seq[r]].long()[js // page_size]
             k = keys[pg, :, js % page_size].float()          # [keys, G, kd]
             v = vals[pg, :, :, js % page_size].float()       # [keys, G, vd]
@@ -337,8 +351,8 @@ class TorchOps:
             out[:, out_offset + h * out_group:out_offset + h * out_group + N] = y[:, h].to(out.dtype)
         return out
 
-    def route_topk(self, z, correction, scale, top):
-        s = torch.softmax(z.float(), dim=-1)
+    def route_topk(self, z, correction, scale, top, score="softmax"):
+        s = torch.sigmoid(z.float()) if score == "sigmoid" else torch.softmax(z.float(), dim=-1)
         choice = s + correction if correction is not None else s
         ids = torch.topk(choice, top, dim=-1).indices
         return ids.to(torch.int32), torch.gather(s, 1, ids) * scale
@@ -360,12 +374,110 @@ class TorchOps:
         own = (ids >= E)[:, :, None]
         return (weights[:, :, None] * torch.where(own, xf[:, None, :], parts.view(n, top, -1))).sum(1)
 
+    def gated_experts(self, x, ids, weights, w_gate_up, w_down, act="silu"):
+        from tiny_inference_server_amd.ops.hip_ops import ChosenExperts
+        E, F = w_gate_up.shape[0], w_gate_up.shape[1] // 2
+        n, top = ids.shape
+        xf = x.float()
+        parts = torch.zeros(n * top, x.shape[1])
+        for r in range(n):
+            for k in range(top):
+                e = int(ids[r, k])
+                z = (w_gate_up[e].float() @ xf[r])[None, :]
+                hid = self.gated_act(z, F, act, row_scale=weights[r, k].reshape(1))[0].float()
+                parts[r * top + k] = w_down[e].float() @ hid
+        return ChosenExperts(parts, ids, None, E, x)
+
+    # ---- blocks whose sublayers read one norm and are summed with a factor per channel ------------------------
+    def dyt32(self, x32, alpha, gain, bias=None):
+        y = torch.tanh(alpha * x32) * gain
+        return (y + bias if bias is not None else y).to(self.dtype)
+
+    def scaled_sum(self, x32, branches, norm=None):
+        from tiny_inference_server_amd.ops.hip_ops import ChosenExperts
+        n = x32.shape[0]
+        total = x32.clone()
+        for y, scale, bias in branches:
+            if isinstance(y, ChosenExperts):
+                top = y.ids.shape[1]
+                w = y.weights[:, :, None] if y.weights is not None else 1.0
+                y = (w * y.results.view(n, top, -1)).sum(1)
+            y = y.float()
+            if bias is not None:
+                y = y + bias
+            total = total + (y * scale if scale is not None else y)
+        x32.copy_(total)
+        normed = self.dyt32(x32, norm[1], norm[2], norm[3]) if norm is not None else None
+        return x32, normed
+
+    def gated_act(self, z, hidden, act, gate_bias=None, up_bias=None, row_scale=None):
+        g, u = z[:, :hidden].float(), z[:, hidden:2 * hidden].float()
+        if gate_bias is not None:
+            g = g + gate_bias
+        if up_bias is not None:
+            u = u + up_bias
+        if row_scale is not None:
+            g, u = g * row_scale[:, None], u * row_scale[:, None]
+        a = torch.nn.functional.gelu(g, approximate="tanh") if act == "gelu_tanh" else g * torch.sigmoid(g)
+        return (a * u).to(self.dtype)
+
+    def softcap(self, z, cap):
+        z.copy_(cap * torch.tanh(z / cap))
+        return z
+
+    # ---- around the scan of a selective state-space mixer ----------------------------------------------------
+    def conv_prepare(self, proj, xbc_off, dt_off, taps, tap_bias, dt_bias, neg_a, state, conv_at, batch, n_heads, vdim):
+        n = proj.shape[0]
+        C, K = taps.shape
+        inner = n_heads * vdim
+        u = torch.zeros(n, C + inner + n_heads, dtype=torch.float32)
+        cu, slots = batch.cu_rows.tolist(), batch.seq_slots.tolist()
+        for k in range(batch.n_seqs):
+            first, rows = cu[k], cu[k + 1] - cu[k]
+            if rows == 0:
+                continue
+            old = state[slots[k], conv_at:conv_at + (K - 1) * C].view(K - 1, C)
+            seq = torch.cat((old, proj[first:first + rows, xbc_off:xbc_off + C].float()), dim=0)
+            acc = (tap_bias if tap_bias is not None else torch.zeros(C)).expand(rows, C).clone()
+            for j in range(K):
+                acc = acc + seq[j:j + rows] * taps[:, j]
+            y = acc * torch.sigmoid(acc)
+            dt = torch.nn.functional.softplus(proj[first:first + rows, dt_off:dt_off + n_heads].float() + dt_bias, threshold=20.0)
+            u[first:first + rows, :C] = y
+            u[first:first + rows, C:C + inner] = (y[:, :inner].view(rows, n_heads, vdim) * dt[:, :, None]).reshape(rows, inner)
+            u[first:first + rows, C + inner:] = torch.exp(neg_a * dt)
+        return u
+
+    def conv_state_update(self, proj, xbc_off, channels, taps, state, conv_at, batch):
+        if taps == 1:
+            return
+        cu, slots = batch.cu_rows.tolist(), batch.seq_slots.tolist()
+        for k in range(batch.n_seqs):
+            first, rows = cu[k], cu[k + 1] - cu[k]
+            if rows == 0:
+                continue
+            line = state[slots[k], conv_at:conv_at + (taps - 1) * channels].view(taps - 1, channels)
+            seq = torch.cat((line, proj[first:first + rows, xbc_off:xbc_off + channels].float()), dim=0)
+            line.copy_(seq[-(taps - 1):])
+
+    def gated_group_norm(self, y, x, skip, vdim, z, gain, eps, parts):
+        n, W = y.shape
+        v = y.float()
+        if skip is not None:
+            v = v + x.float() * skip.repeat_interleave(vdim)
+        if z is not None:
+            zf = z.float()
+            v = v * zf * torch.sigmoid(zf)
+        v = v.view(n, parts, W // parts)
+        v = (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)).reshape(n, W) * gain
+        return v.to(self.dtype)
+
     @staticmethod
     def state_scan_floats(kind, n_heads, dim, vdim):
         return n_heads * dim * vdim + (n_heads * -(-vdim // 16) * (dim + 1) if kind == "gated_max" else 0)
 
     def state_scan(self, kind, proj, q_off, k_off, v_off, q_scale, state, batch, n_heads, dim, vdim, decay=None,
-                   i_off=0, f_off=0, bias_i=None, bias_f=None, cap=0.0):
+                   i_off=0, f_off=0, bias_i=None, bias_f=None, cap=0.0, qk_group=1, decay_per_head=False):
         """The same line of state as the kernel keeps (n and m once per block of 16 value channels)."""
         n, H, D, V = proj.shape[0], n_heads, dim, vdim
         blocks = -(-V // 16)
@@ -380,11 +492,13 @@ class TorchOps:
             S = line[:H * D * V].view(H, D, V)
             nm = line[H * D * V:H * D * V + H * blocks * (D + 1)].view(H, blocks, D + 1) if kind == "gated_max" else None
             for r in range(first, first + rows):
-                q = proj[r, q_off:q_off + H * D].float().view(H, D) * q_scale
-                kk = proj[r, k_off:k_off + H * D].float().view(H, D)
+                Hq = H // qk_group
+                q = proj[r, q_off:q_off + Hq * D].float().view(Hq, D).repeat_interleave(qk_group, dim=0) * q_scale
+                kk = proj[r, k_off:k_off + Hq * D].float().view(Hq, D).repeat_interleave(qk_group, dim=0)
                 v = proj[r, v_off:v_off + H * V].float().view(H, V)
                 if kind == "decay":
-                    S.copy_(decay[r].view(H, D, 1) * S + kk[:, :, None] * v[:, None, :])
+                    a = decay[r, :H].view(H, 1, 1) if decay_per_head else decay[r].view(H, D, 1)
+                    S.copy_(a * S + kk[:, :, None] * v[:, None, :])
                     o = torch.einsum("hdv,hd->hv", S, q)
                 else:
                     gi = cap * torch.tanh((proj[r, i_off:i_off + H].float() + bias_i) / cap)

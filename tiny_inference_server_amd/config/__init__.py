@@ -3,3 +3,4 @@ from .model_config import (ARCHITECTURES, Architecture, ConfigError, GqaMtpConfi
 from .registry import Registry
 from .fikevik_config import FikevikConfig
 from .fipuzen_config import FipuzenConfig
+from .rurorax_config import RuroraxConfig

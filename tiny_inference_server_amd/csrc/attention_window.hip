@@ -7,7 +7,8 @@
 // A page of `page_size` slots holds, for each key/value head, the keys as [slot][key size] and then, after the keys
 // of all heads, the values transposed as [value size][slot]. With equal sizes that is the layout the other attention
 // kernels read. The row at position p sees
-// the keys at [max(0, p - window + 1), p] (window 0: all), found through the request's block table; keys outside are
+// the keys at [max(0, p - window + 1), p] (window 0: all), and with chunk_size c > 0 only those from p - p % c on (the
+// row's own chunk of positions, chunks counted from position 0), found through the request's block table; keys outside are
 // never read, so what a reused page holds cannot reach a result.
 // Norms, angles, scores, the softmax and the weighted sum are 32-bit; `T` is the type of queries and pages.
 #include "common.h"
@@ -33,8 +34,12 @@ struct PrepareArgs {
   int value_norm;          // values are divided by their root mean square
   float temp_coef;         // queries times 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1); 0: none
   int temp_every;
+  int whole_norm;          // the norms run over all heads of a row's queries (keys) at once, with gains of [H * KD] ([G * KD])
+  int pair_half;           // rotated pairs are (i, i + rot_dims / 2) instead of (2i, 2i + 1)
 };
 
+// The norms may also run over all heads of a row at once (whole_norm), and the rotated pairs may be (i, i + rot_dims/2)
+// (pair_half).
 // grid (rows, H + 2 G), one wave each: unit u < H is a query head, u < H + G a key head, else a value head.
 // proj holds the projections of a row in 32-bit: queries at q_off, keys at k_off, values at v_off.
 template <typename T>
@@ -54,7 +59,20 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
     if (bias) bias += (long)h * KD;
     const float* gain = is_q ? a.q_gain : a.k_gain;
     float inv = 1.f;
-    if (gain) {
+    if (gain && a.whole_norm) {
+      // every head's wave sums the whole projection, in the same order: lanes over the channels, then the wave
+      const int n_all = (is_q ? H : G) * KD;
+      const float* all = proj + r * ldp + (is_q ? q_off : k_off);
+      const float* all_bias = is_q ? a.q_bias : a.k_bias;
+      float ss = 0.f;
+      for (int e = lane; e < n_all; e += TIS_WAVE) {
+        const float v = all[e] + (all_bias ? all_bias[e] : 0.f);
+        ss += v * v;
+      }
+      ss = wave_sum(ss);
+      inv = 1.f / sqrtf(ss / (float)n_all + a.eps);
+      gain += (long)h * KD;
+    } else if (gain) {
       float ss = 0.f;
       for (int e = lane; e < KD; e += TIS_WAVE) {
         const float v = src[e] + (bias ? bias[e] : 0.f);
@@ -74,6 +92,20 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
       const int ws = write_slots[r];
       dst = plane + (long)(ws / page_size) * page_stride + ((long)h * page_size + ws % page_size) * KD;
     }
+    if (a.pair_half) {
+      const int half = a.rot_dims / 2;
+      for (int p = lane; p < half; p += TIS_WAVE) {
+        const int e0 = p, e1 = p + half;
+        const float x = (src[e0] + (bias ? bias[e0] : 0.f)) * inv * (gain ? gain[e0] : 1.f);
+        const float y = (src[e1] + (bias ? bias[e1] : 0.f)) * inv * (gain ? gain[e1] : 1.f);
+        float sn, cs;
+        sincosf(pos * a.freqs[p], &sn, &cs);
+        dst[e0] = from_f<T>((x * cs - y * sn) * factor);
+        dst[e1] = from_f<T>((y * cs + x * sn) * factor);
+      }
+      for (int e = a.rot_dims + lane; e < KD; e += TIS_WAVE)
+        dst[e] = from_f<T>((src[e] + (bias ? bias[e] : 0.f)) * inv * (gain ? gain[e] : 1.f) * factor);
+    } else
     for (int p = lane; 2 * p < KD; p += TIS_WAVE) {
       const int e0 = 2 * p, e1 = e0 + 1;
       float x = (src[e0] + (bias ? bias[e0] : 0.f)) * inv * (gain ? gain[e0] : 1.f);
@@ -175,7 +207,8 @@ template <typename T>
 __global__ __launch_bounds__(AW_THREADS) void attention_window_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ plane, const int* __restrict__ block_tables, int bt_ld,
     const int* __restrict__ row_seq, const int* __restrict__ positions, T* __restrict__ out, long ldo, int group_size,
-    int G, int KD, int VD, int page_size, int window, float scale, int sink, const float* __restrict__ gate, long ldg) {
+    int G, int KD, int VD, int page_size, int window, int chunk_size, float scale, int sink,
+    const float* __restrict__ gate, long ldg) {
   __shared__ float qs[AW_MAX_DIM];
   __shared__ float sc[AW_CHUNK];
   __shared__ float red[16];
@@ -184,7 +217,8 @@ __global__ __launch_bounds__(AW_THREADS) void attention_window_kernel(
   const int h = blockIdx.y, g = h / group_size, t = threadIdx.x;
   const int pos = positions[r];
   const int* bt = block_tables + (long)row_seq[r] * bt_ld;
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  if (chunk_size > 0) first = max(first, pos - pos % chunk_size);     // only keys of the row's own chunk of positions
   const int end = pos + 1;
   for (int d = t; d < KD; d += AW_THREADS) qs[d] = to_f(q[r * ldq + (long)h * KD + d]) * scale;
   __syncthreads();
@@ -254,8 +288,8 @@ TIS_EXPORT int tis_attention_prepare(int dtype, const float* proj, long ldp, int
                                      const int* positions, const int* write_slots, void* plane, void* q_out, long ldq,
                                      const float* q_bias, const float* k_bias, const float* v_bias, const float* q_gain,
                                      const float* k_gain, const float* q_factor, const float* freqs, int rot_dims, float eps,
-                                     int value_norm, float temp_coef, int temp_every, int rows, int H, int G, int KD, int VD,
-                                     int page_size, hipStream_t stream) {
+                                     int value_norm, float temp_coef, int temp_every, int whole_norm, int pair_half, int rows,
+                                     int H, int G, int KD, int VD, int page_size, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || H < 1 || G < 1 || KD < 1 || VD < 1 || page_size < 1 || H + 2 * G > 65535)
     return tis_fail("attention_prepare: bad size rows=%d heads=%d kv_heads=%d key=%d value=%d page=%d", rows, H, G, KD, VD,
@@ -264,7 +298,8 @@ TIS_EXPORT int tis_attention_prepare(int dtype, const float* proj, long ldp, int
     return tis_fail("attention_prepare: %d rotated channels of %d", rot_dims, KD);
   if (temp_coef != 0.f && temp_every < 1) return tis_fail("attention_prepare: a query factor every %d positions", temp_every);
   if (write_slots && !plane) return tis_fail("attention_prepare: write slots without pages");
-  PrepareArgs a{q_bias, k_bias, v_bias, q_gain, k_gain, q_factor, freqs, rot_dims, eps, value_norm, temp_coef, temp_every};
+  PrepareArgs a{q_bias, k_bias, v_bias, q_gain, k_gain, q_factor, freqs, rot_dims, eps, value_norm, temp_coef, temp_every,
+                whole_norm, pair_half};
   dim3 grid(rows, H + 2 * G);
   if (dtype == TIS_F32)
     attention_prepare_kernel<float><<<grid, TIS_WAVE, 0, stream>>>(proj, ldp, q_off, k_off, v_off, positions, write_slots,
@@ -301,20 +336,20 @@ TIS_EXPORT int tis_latent_prepare(int dtype, const float* proj, long ldp, int q_
 
 TIS_EXPORT int tis_attention_window(int dtype, const void* q, long ldq, const void* plane, const int* block_tables,
                                     int bt_ld, const int* row_seq, const int* positions, void* out, long ldo, int rows,
-                                    int H, int G, int KD, int VD, int page_size, int window, float scale, int sink,
-                                    const float* gate, long ldg, hipStream_t stream) {
+                                    int H, int G, int KD, int VD, int page_size, int window, int chunk_size, float scale,
+                                    int sink, const float* gate, long ldg, hipStream_t stream) {
   if (rows == 0) return 0;
-  if (rows < 0 || H < 1 || G < 1 || H % G || page_size < 1 || window < 0 || H > 65535)
+  if (rows < 0 || H < 1 || G < 1 || H % G || page_size < 1 || window < 0 || chunk_size < 0 || H > 65535)
     return tis_fail("attention_window: bad size rows=%d heads=%d kv_heads=%d page=%d window=%d", rows, H, G, page_size, window);
   if (KD < 1 || KD > AW_MAX_DIM || VD < 1 || VD > AW_MAX_DIM)
     return tis_fail("attention_window: key size %d or value size %d is outside 1..%d", KD, VD, AW_MAX_DIM);
   dim3 grid(rows, H);
   if (dtype == TIS_F32)
     attention_window_kernel<float><<<grid, AW_THREADS, 0, stream>>>((const float*)q, ldq, (const float*)plane, block_tables,
-        bt_ld, row_seq, positions, (float*)out, ldo, H / G, G, KD, VD, page_size, window, scale, sink, gate, ldg);
+        bt_ld, row_seq, positions, (float*)out, ldo, H / G, G, KD, VD, page_size, window, chunk_size, scale, sink, gate, ldg);
   else if (dtype == TIS_BF16)
     attention_window_kernel<bf16><<<grid, AW_THREADS, 0, stream>>>((const bf16*)q, ldq, (const bf16*)plane, block_tables,
-        bt_ld, row_seq, positions, (bf16*)out, ldo, H / G, G, KD, VD, page_size, window, scale, sink, gate, ldg);
+        bt_ld, row_seq, positions, (bf16*)out, ldo, H / G, G, KD, VD, page_size, window, chunk_size, scale, sink, gate, ldg);
   else
     return tis_fail("unknown dtype code %d", dtype);
   return tis_launch_status("attention_window");

@@ -29,7 +29,7 @@ __device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.f + 
 // one wave per row
 __global__ __launch_bounds__(TIS_WAVE) void route_topk_kernel(const float* __restrict__ z, long ldz,
                                                               const float* __restrict__ correction, float scale,
-                                                              int n_out, int top, int* __restrict__ ids,
+                                                              int n_out, int top, int score, int* __restrict__ ids,
                                                               float* __restrict__ weights) {
   const long r = blockIdx.x;
   const int lane = threadIdx.x;
@@ -46,11 +46,12 @@ __global__ __launch_bounds__(TIS_WAVE) void route_topk_kernel(const float* __res
 #pragma unroll
   for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
     const int e = lane + u * TIS_WAVE;
-    s[u] = e < n_out ? expf(s[u] - m) : 0.f;
+    if (score == 1) s[u] = e < n_out ? 1.f / (1.f + expf(-s[u])) : 0.f;      // a sigmoid per output, no sum over them
+    else s[u] = e < n_out ? expf(s[u] - m) : 0.f;
     sum += s[u];
   }
   sum = wave_sum(sum);
-  const float inv = 1.f / sum;
+  const float inv = score == 1 ? 1.f : 1.f / sum;
 #pragma unroll
   for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
     const int e = lane + u * TIS_WAVE;
@@ -369,12 +370,13 @@ __global__ __launch_bounds__(256) void experts_combine_kernel(const float* __res
   }
 }
 
-TIS_EXPORT int tis_route_topk(const float* z, long ldz, const float* correction, float scale, int rows, int n_out, int top,
+TIS_EXPORT int tis_route_topk(const float* z, long ldz, const float* correction, float scale, int rows, int n_out, int top, int score,
                               int* ids, float* weights, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || n_out < 1 || n_out > EX_MAX_PER_LANE * TIS_WAVE || top < 1 || top > n_out)
     return tis_fail("route_topk: bad size rows=%d outputs=%d (at most %d) top=%d", rows, n_out, EX_MAX_PER_LANE * TIS_WAVE, top);
-  route_topk_kernel<<<rows, TIS_WAVE, 0, stream>>>(z, ldz, correction, scale, n_out, top, ids, weights);
+  if (score != 0 && score != 1) return tis_fail("route_topk: score kind %d (0: softmax, 1: sigmoid)", score);
+  route_topk_kernel<<<rows, TIS_WAVE, 0, stream>>>(z, ldz, correction, scale, n_out, top, score, ids, weights);
   return tis_launch_status("route_topk");
 }
 

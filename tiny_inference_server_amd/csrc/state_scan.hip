@@ -41,6 +41,13 @@ __device__ __forceinline__ float sc_log_sigmoid(float z) { return fminf(z, 0.f) 
 //                                   start in their place and the m at its start into the last float
 //   cum       [row][H*D]            kind 0: product of the decays from the segment's start to the row
 //   aux       [row][H][3]           kind 1: m', F and n . q of the segment alone
+// Where a head finds its columns: `qk_group` consecutive heads share one set of query and key columns (1: every head
+// has its own); head h's decay for key channel i lies at h * decay_hs + i * decay_cs of a row's decays (D and 1: one per
+// key channel; 1 and 0: one per head).
+struct ScanLayout {
+  int qk_group, decay_hs, decay_cs;
+};
+
 struct SegArgs {
   int segments;      // most segments of one request in this call; 0: not segmented
   int seg_len;
@@ -58,7 +65,7 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
     const float* __restrict__ decay, long ldd, int i_off, int f_off, const float* __restrict__ bias_i,
     const float* __restrict__ bias_f, float cap, float* __restrict__ state, long state_ld,
     const int* __restrict__ cu_rows, const int* __restrict__ seq_slots, float* __restrict__ out, long ldo, int H, int D,
-    int V, int n_vb, int chunk, SegArgs sg) {
+    int V, int n_vb, int chunk, SegArgs sg, ScanLayout lay) {
   static_assert(SEG || VB == SC_VB, "a state line keeps n and m per 16 value channels");
   constexpr int R = SC_THREADS / VB;
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -102,9 +109,9 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
       const int c = idx / DP, i = idx - c * DP;
       const float* row = proj + (long)(c0 + c) * ldp;
       const bool in = i < D;
-      sq[idx] = in ? row[q_off + h * D + i] * q_scale : 0.f;
-      sk[idx] = in ? row[k_off + h * D + i] : 0.f;
-      if (KIND == 0) sa[idx] = in ? decay[(long)(c0 + c) * ldd + h * D + i] : 0.f;
+      sq[idx] = in ? row[q_off + (h / lay.qk_group) * D + i] * q_scale : 0.f;
+      sk[idx] = in ? row[k_off + (h / lay.qk_group) * D + i] : 0.f;
+      if (KIND == 0) sa[idx] = in ? decay[(long)(c0 + c) * ldd + h * lay.decay_hs + i * lay.decay_cs] : 0.f;
     }
     for (int idx = t; idx < nc * VB; idx += SC_THREADS) {
       const int c = idx / VB, jj = idx - c * VB;
@@ -249,7 +256,7 @@ template <int KIND>
 __global__ __launch_bounds__(SC_THREADS) void segment_outputs_kernel(const float* __restrict__ proj, long ldp, int q_off,
                                                                      float q_scale, const int* __restrict__ cu_rows,
                                                                      float* __restrict__ out, long ldo, int H, int D,
-                                                                     int V, SegArgs sg) {
+                                                                     int V, SegArgs sg, ScanLayout lay) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* s0 = lds;                       // [D][SG_COLS]
   float* qt = s0 + D * SG_COLS;          // [SG_ROWS][D + 1]
@@ -270,7 +277,7 @@ __global__ __launch_bounds__(SC_THREADS) void segment_outputs_kernel(const float
     __syncthreads();
     for (int idx = t; idx < nr * D; idx += SC_THREADS) {
       const int r = idx / D, i = idx - r * D;
-      float q = proj[(long)(t0 + r) * ldp + q_off + h * D + i] * q_scale;
+      float q = proj[(long)(t0 + r) * ldp + q_off + (h / lay.qk_group) * D + i] * q_scale;
       if (KIND == 0) q *= sg.cum[(long)(t0 + r) * H * D + h * D + i];
       qt[r * (D + 1) + i] = q;
     }
@@ -315,20 +322,21 @@ template <int KIND>
 static int launch_scan(bool wide, int ns, dim3 grid, size_t lds, hipStream_t stream, const float* proj, long ldp, int q_off, int k_off,
                        int v_off, float q_scale, const float* decay, long ldd, int i_off, int f_off, const float* bias_i,
                        const float* bias_f, float cap, float* state, long state_ld, const int* cu_rows,
-                       const int* seq_slots, float* out, long ldo, int H, int D, int V, int n_vb, int chunk, SegArgs sg) {
+                       const int* seq_slots, float* out, long ldo, int H, int D, int V, int n_vb, int chunk, SegArgs sg,
+                       ScanLayout lay) {
 #define SC_LAUNCH(NS)                                                                                                   \
   if (sg.segments)                                                                                                      \
     state_scan_kernel<KIND, NS, true, SC_VB><<<grid, SC_THREADS, lds, stream>>>(                                        \
         proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off, bias_i, bias_f, cap, state, state_ld,        \
-        cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);                                                        \
+        cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg, lay);                                                   \
   else                                                                                                                  \
     state_scan_kernel<KIND, NS, false, SC_VB><<<grid, SC_THREADS, lds, stream>>>(                                       \
         proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off, bias_i, bias_f, cap, state, state_ld,        \
-        cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg)
+        cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg, lay)
 #define SC_LAUNCH_WIDE(NS)                                                                                              \
   state_scan_kernel<KIND, NS, true, SC_WIDE_VB><<<grid, SC_THREADS, lds, stream>>>(                                     \
       proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off, bias_i, bias_f, cap, state, state_ld, cu_rows, \
-      seq_slots, out, ldo, H, D, V, n_vb, chunk, sg)
+      seq_slots, out, ldo, H, D, V, n_vb, chunk, sg, lay)
   if (wide) {
     if (ns <= 8) { SC_LAUNCH_WIDE(8); }
     else if (ns <= 16) { SC_LAUNCH_WIDE(16); }
@@ -350,7 +358,7 @@ static int launch_scan(bool wide, int ns, dim3 grid, size_t lds, hipStream_t str
   if (tis_launch_status("segment_states")) return -1;
   const size_t lds3 = sizeof(float) * ((size_t)D * SG_COLS + (size_t)SG_ROWS * (D + 1) + SG_ROWS);
   segment_outputs_kernel<KIND><<<dim3(grid.x, H, (V + SG_COLS - 1) / SG_COLS), SC_THREADS, lds3, stream>>>(
-      proj, ldp, q_off, q_scale, cu_rows, out, ldo, H, D, V, sg);
+      proj, ldp, q_off, q_scale, cu_rows, out, ldo, H, D, V, sg, lay);
   return tis_launch_status("segment_outputs");
 }
 
@@ -374,8 +382,11 @@ TIS_EXPORT int tis_state_scan(int kind, const float* proj, long ldp, int q_off, 
                               const float* decay, long ldd, int i_off, int f_off, const float* bias_i,
                               const float* bias_f, float cap, float* state, long state_ld, const int* cu_rows,
                               const int* seq_slots, int n_seqs, float* out, long ldo, int H, int D, int V,
-                              int segments, int seg_len, int rows, float* workspace, hipStream_t stream) {
+                              int segments, int seg_len, int rows, float* workspace, int qk_group, int decay_per_head,
+                              hipStream_t stream) {
   if (n_seqs == 0) return 0;
+  if (qk_group < 1 || H % qk_group) return tis_fail("state_scan: %d heads in groups of %d", H, qk_group);
+  const ScanLayout lay = {qk_group, decay_per_head ? 1 : D, decay_per_head ? 0 : 1};
   if (n_seqs < 0 || H < 1 || H > 65535 || D < 1 || D > SC_R * 16 || V < 1)
     return tis_fail("state_scan: bad size requests=%d heads=%d key channels=%d (at most %d) value channels=%d", n_seqs, H,
                     D, SC_R * 16, V);
@@ -417,7 +428,7 @@ TIS_EXPORT int tis_state_scan(int kind, const float* proj, long ldp, int q_off, 
   const int ns = ns_need;
   if (kind == 0)
     return launch_scan<0>(wide, ns, grid, bytes(chunk), stream, proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off,
-                          bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);
+                          bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg, lay);
   return launch_scan<1>(wide, ns, grid, bytes(chunk), stream, proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off,
-                        bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);
+                        bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg, lay);
 }

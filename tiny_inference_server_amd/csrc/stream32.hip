@@ -443,3 +443,132 @@ TIS_EXPORT int tis_head_gate(int dtype, void* x, long ldx, const float* gate, lo
                (head_gate_kernel<bf16><<<blocks, S32_THREADS, 0, stream>>>((bf16*)x, ldx, gate, ldg, rows, H, V)))
   return tis_launch_status("head_gate");
 }
+
+// ---- blocks whose sublayers all read one norm of the stream and are summed with a factor per channel ---------------
+
+// Dynamic tanh: out = tanh(alpha * x) * gain + bias, element by element (no mean, no variance), in the compute type.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void dyt32_kernel(const float* __restrict__ x, float alpha,
+                                                             const float* __restrict__ gain, const float* __restrict__ bias,
+                                                             T* __restrict__ out, long ldo, int D) {
+  const long r = blockIdx.x;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS)
+    out[r * ldo + c] = from_f<T>(tanhf(alpha * x[r * D + c]) * gain[c] + (bias ? bias[c] : 0.f));
+}
+
+// One branch of a scaled sum: s[c] * (y[r][c] + b[c]); s and b may be null (1 and 0). With `cs.ids` the branch is the
+// not yet summed result of a routed feed-forward (see ChosenSum; weights may be null: every choice counts once).
+struct ScaledBranch {
+  const float* y;
+  long ld;
+  const float* scale;
+  const float* bias;
+};
+
+// x <- x + sum over the branches, in place or into out32; `normed` (nullable) gets the dynamic tanh of the new row in
+// the compute type (the norm that the next block, or the model's end, reads the stream through).
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void scaled_sum_kernel(const float* __restrict__ x, ScaledBranch a, ScaledBranch b,
+                                                                  ChosenSum cs, float* __restrict__ out32, int norm_kind,
+                                                                  float alpha, const float* __restrict__ gain,
+                                                                  const float* __restrict__ nbias, T* __restrict__ normed,
+                                                                  long ldn, int D) {
+  const long r = blockIdx.x;
+  __shared__ int chosen_id[64];
+  __shared__ float chosen_w[64];
+  const bool kept = cs.ids && cs.top <= 64;
+  if (kept) {
+    if (threadIdx.x < cs.top) {
+      chosen_id[threadIdx.x] = cs.ids[r * cs.top + threadIdx.x];
+      chosen_w[threadIdx.x] = cs.weights ? cs.weights[r * cs.top + threadIdx.x] : 1.f;
+    }
+    __syncthreads();
+  }
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    float v = x[r * D + c];
+    if (a.y) v += (a.scale ? a.scale[c] : 1.f) * (a.y[r * a.ld + c] + (a.bias ? a.bias[c] : 0.f));
+    if (cs.ids) {
+      float y = 0.f;
+      for (int k = 0; k < cs.top; ++k) {
+        const int e = kept ? chosen_id[k] : cs.ids[r * cs.top + k];
+        const float w = kept ? chosen_w[k] : (cs.weights ? cs.weights[r * cs.top + k] : 1.f);
+        y += w * (e < cs.n_experts ? b.y[(r * cs.top + k) * b.ld + c] : to_f(static_cast<const T*>(cs.rows)[r * cs.ldr + c]));
+      }
+      v += (b.scale ? b.scale[c] : 1.f) * (y + (b.bias ? b.bias[c] : 0.f));
+    } else if (b.y) {
+      v += (b.scale ? b.scale[c] : 1.f) * (b.y[r * b.ld + c] + (b.bias ? b.bias[c] : 0.f));
+    }
+    out32[r * D + c] = v;
+    if (norm_kind == 3) normed[r * ldn + c] = from_f<T>(tanhf(alpha * v) * gain[c] + (nbias ? nbias[c] : 0.f));
+  }
+}
+
+// out[r][j] = act(w_r * (z[r][j] + gb[j])) * (w_r * (z[r][F + j] + ub[j])): the gate of a gated feed-forward on a
+// 32-bit product whose first F columns are the gate's and whose next F the other factor's. Biases and the factor per
+// row (a router's weight on the row that an expert read) may be null. act 0: tanh-form gelu, 1: silu.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void gated_act_kernel(const float* __restrict__ z, long ldz, int F,
+                                                                 const float* __restrict__ gb, const float* __restrict__ ub,
+                                                                 const float* __restrict__ row_scale, int act,
+                                                                 T* __restrict__ out, long ldo, int rows) {
+  const long i = (long)blockIdx.x * S32_THREADS + threadIdx.x;
+  if (i >= (long)rows * F) return;
+  const long r = i / F;
+  const int j = (int)(i % F);
+  const float w = row_scale ? row_scale[r] : 1.f;
+  const float g = w * (z[r * ldz + j] + (gb ? gb[j] : 0.f)), u = w * (z[r * ldz + F + j] + (ub ? ub[j] : 0.f));
+  out[r * ldo + j] = from_f<T>((act == 0 ? gelu_tanh_f(g) : g * sigmoid_f(g)) * u);
+}
+
+// z <- cap * tanh(z / cap) on 32-bit rows, in place
+__global__ __launch_bounds__(S32_THREADS) void softcap_kernel(float* __restrict__ z, long ldz, float cap, int rows, int W) {
+  const long i = (long)blockIdx.x * S32_THREADS + threadIdx.x;
+  if (i >= (long)rows * W) return;
+  float* p = z + (i / W) * ldz + (i % W);
+  *p = cap * tanhf(*p / cap);
+}
+
+TIS_EXPORT int tis_dyt32(int dtype, const float* x, float alpha, const float* gain, const float* bias, void* out, long ldo,
+                         int rows, int D, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1 || !x || !gain || !out) return tis_fail("dyt32: bad arguments rows=%d width=%d", rows, D);
+  S32_DISPATCH((dyt32_kernel<float><<<rows, S32_THREADS, 0, stream>>>(x, alpha, gain, bias, (float*)out, ldo, D)),
+               (dyt32_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>(x, alpha, gain, bias, (bf16*)out, ldo, D)))
+  return tis_launch_status("dyt32");
+}
+
+TIS_EXPORT int tis_scaled_sum(int dtype, const float* x, const float* y0, long ld0, const float* s0, const float* b0,
+                              const float* y1, long ld1, const float* s1, const float* b1, const int* ids,
+                              const float* weights, int top, int n_experts, const void* chosen_rows, long ldr,
+                              float* out32, int norm_kind, float alpha, const float* gain, const float* nbias, void* normed,
+                              long ldn, int rows, int D, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1 || !x || !out32) return tis_fail("scaled_sum: bad arguments rows=%d width=%d", rows, D);
+  if (ids && (top < 1 || n_experts < 0 || (n_experts > 0 && !y1) || !chosen_rows))
+    return tis_fail("scaled_sum: a sum over chosen experts needs ids, the experts' results and the rows they read");
+  if ((norm_kind != 0 && norm_kind != 3) || (norm_kind && (!gain || !normed)))
+    return tis_fail("scaled_sum: norm kind %d (0: none, 3: dynamic tanh, with a gain and an output)", norm_kind);
+  const ScaledBranch a{y0, ld0, s0, b0}, b{y1, ld1, s1, b1};
+  const ChosenSum cs{ids, weights, top, n_experts, chosen_rows, ldr};
+  S32_DISPATCH((scaled_sum_kernel<float><<<rows, S32_THREADS, 0, stream>>>(x, a, b, cs, out32, norm_kind, alpha, gain, nbias, (float*)normed, ldn, D)),
+               (scaled_sum_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>(x, a, b, cs, out32, norm_kind, alpha, gain, nbias, (bf16*)normed, ldn, D)))
+  return tis_launch_status("scaled_sum");
+}
+
+TIS_EXPORT int tis_gated_act(int dtype, const float* z, long ldz, int F, const float* gate_bias, const float* up_bias,
+                             const float* row_scale, int act, void* out, long ldo, int rows, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || F < 1 || (act != 0 && act != 1)) return tis_fail("gated_act: bad size rows=%d hidden=%d act=%d", rows, F, act);
+  const long blocks = ((long)rows * F + S32_THREADS - 1) / S32_THREADS;
+  S32_DISPATCH((gated_act_kernel<float><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, F, gate_bias, up_bias, row_scale, act, (float*)out, ldo, rows)),
+               (gated_act_kernel<bf16><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, F, gate_bias, up_bias, row_scale, act, (bf16*)out, ldo, rows)))
+  return tis_launch_status("gated_act");
+}
+
+TIS_EXPORT int tis_softcap(float* z, long ldz, float cap, int rows, int W, hipStream_t stream) {
+  if (rows == 0 || W == 0) return 0;
+  if (rows < 0 || W < 0 || !(cap > 0.f)) return tis_fail("softcap: bad arguments rows=%d width=%d cap=%g", rows, W, (double)cap);
+  const long blocks = ((long)rows * W + S32_THREADS - 1) / S32_THREADS;
+  softcap_kernel<<<blocks, S32_THREADS, 0, stream>>>(z, ldz, cap, rows, W);
+  return tis_launch_status("softcap");
+}

@@ -154,7 +154,8 @@ class Model:
 
     def _project(self, rows):
         """Rows after a stage's closing norm -> 32-bit logits: the one place the output table is applied."""
-        return self.ops.linear(rows, self.shared["lm_head"], out_dtype=torch.float32)
+        logits = self.ops.linear(rows, self.shared["lm_head"], out_dtype=torch.float32)
+        return self.ops.softcap(logits, self.spec.logit_softcap) if self.spec.logit_softcap else logits
 
     def logits(self, hidden, want_index, n):
         """32-bit logits [n, vocab] of the rows `want_index` of `hidden` (reference main_models_new.py:225-226)."""

@@ -45,6 +45,7 @@ SOURCES: Dict[str, str] = {
     "state_scan": "state_scan.hip",
     "experts": "experts.hip",
     "attention_latent": "attention_latent.hip",
+    "ssm_parts": "ssm_parts.hip",
 }
 HEADERS = ["common.h", "attention_mfma.h"]
 # what a library links beyond the HIP runtime

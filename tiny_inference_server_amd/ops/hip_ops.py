@@ -114,25 +114,35 @@ _SIGNATURES["stream32"] = ("tis_stream32", {
     "tis_gate_table": [_I, _P, _L, _P, _L, _P, _I, _P, _L, _I, _I, _P],
     "tis_activate32": [_P, _L, _I, _I, _I, _P],
     "tis_head_gate": [_I, _P, _L, _P, _L, _I, _I, _I, _P],
+    "tis_dyt32": [_I, _P, _F, _P, _P, _P, _L, _I, _I, _P],
+    "tis_scaled_sum": [_I, _P, _P, _L, _P, _P, _P, _L, _P, _P, _P, _P, _I, _I, _P, _L, _P, _I, _F, _P, _P, _P, _L, _I, _I,
+                       _P],
+    "tis_gated_act": [_I, _P, _L, _I, _P, _P, _P, _I, _P, _L, _I, _P],
+    "tis_softcap": [_P, _L, _F, _I, _I, _P],
 })
 _SIGNATURES["attention_window"] = ("tis_attention_window", {
     "tis_attention_prepare": [_I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _F, _I,
-                              _I, _I, _I, _I, _I, _I, _P],
+                              _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "tis_latent_prepare": [_I, _P, _L, _I, _I, _P, _P, _P, _P, _L, _P, _L, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P],
-    "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _P],
+    "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _P],
 })
 _SIGNATURES["attention_latent"] = ("tis_attention_latent", {
     "tis_attention_latent": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
 })
 _SIGNATURES["experts"] = ("tis_experts", {
-    "tis_route_topk": [_P, _L, _P, _F, _I, _I, _I, _P, _P, _P],
+    "tis_route_topk": [_P, _L, _P, _F, _I, _I, _I, _I, _P, _P, _P],
     "tis_expert_lists": [_P, _I, _I, _I, _P, _P, _P],
     "tis_grouped_linear": [_I, _I, _P, _L, _L, _I, _P, _P, _L, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "tis_experts_combine": [_I, _P, _L, _P, _L, _P, _P, _I, _I, _P, _L, _I, _I, _P],
 })
 _SIGNATURES["state_scan"] = ("tis_state_scan", {
     "tis_state_scan": [_I, _P, _L, _I, _I, _I, _F, _P, _L, _I, _I, _P, _P, _F, _P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _I,
-                       _I, _I, _P, _P],
+                       _I, _I, _P, _I, _I, _P],
+})
+_SIGNATURES["ssm_parts"] = ("tis_ssm", {
+    "tis_conv_prepare": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _L, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P],
+    "tis_conv_state_update": [_P, _L, _I, _P, _L, _I, _P, _P, _I, _I, _I, _P],
+    "tis_gated_group_norm": [_I, _P, _L, _P, _L, _P, _I, _P, _L, _P, _F, _P, _L, _I, _I, _I, _P],
 })
 
 _libs = {}
@@ -1266,6 +1276,164 @@ class HipOps:
         self._lazy("stream32").tis_activate32(_ptr(z), z.stride(0), self._ACTS[act], z.shape[0], z.shape[1], self._stream())
         return z
 
+    # ---- blocks whose sublayers read one norm of the stream and are summed with a factor per channel --------------
+    def dyt32(self, x32, alpha: float, gain, bias=None):
+        """Dynamic tanh of 32-bit rows, tanh(alpha * x) * gain + bias element by element, in the compute type."""
+        n, D = x32.shape
+        self._f32(x32, "dyt32 x", n * D)
+        self._f32(gain, "dyt32 gain", D)
+        if bias is not None:
+            self._f32(bias, "dyt32 bias", D)
+        out = self.empty(n, D)
+        self._lazy("stream32").tis_dyt32(self.code, _ptr(x32), float(alpha), _ptr(gain), _ptr(bias), _ptr(out), out.stride(0),
+                                         n, D, self._stream())
+        return out
+
+    def scaled_sum(self, x32, branches, norm=None):
+        """x32 <- x32 + sum_i scale_i * (y_i + bias_i), in place: (x32, normed). branches: one or two (y, scale, bias)
+        with y [rows, width] 32-bit (a strided view is fine), scale and bias [width] 32-bit or None (1 and 0). The
+        second y may be a `ChosenExperts` (a routed feed-forward's results before the sum over a row's choices, which is
+        then taken here; weights None: every choice counts once). norm = ("dyt", alpha, gain, bias): also return the
+        dynamic tanh of the new rows in the compute type."""
+        n, D = x32.shape
+        self._f32(x32, "scaled_sum x", n * D)
+        if not 1 <= len(branches) <= 2:
+            raise KernelError(f"scaled_sum: {len(branches)} branches (one or two)")
+        chosen = None
+        args = []
+        for i, (y, scale, bias) in enumerate(branches):
+            if isinstance(y, ChosenExperts):
+                if i == 0:
+                    raise KernelError("scaled_sum: a routed feed-forward's results come as the second branch")
+                chosen, y = y, y.results
+                top = chosen.ids.shape[1]
+                self._index(chosen.ids, "expert ids", n * top)
+                if chosen.weights is not None:
+                    self._f32(chosen.weights, "expert weights", n * top)
+                _rows_view(self._check(chosen.rows, "experts' input rows"), "experts' input rows")
+                if tuple(chosen.rows.shape) != (n, D):
+                    raise KernelError(f"scaled_sum: experts' input rows {tuple(chosen.rows.shape)} for {n} rows of {D}")
+                if y is not None:
+                    self._f32_rows(y, "experts' results", n * top, D)
+            else:
+                self._f32_rows(y, "scaled_sum branch", n, D)
+            for t, what in ((scale, "scaled_sum factors"), (bias, "scaled_sum bias")):
+                if t is not None:
+                    self._f32(t, what, D)
+            args += [_ptr(y), y.stride(0) if y is not None else 0, _ptr(scale), _ptr(bias)]
+        if len(branches) == 1:
+            args += [_ptr(None), 0, _ptr(None), _ptr(None)]
+        kind, alpha, gain, nbias, normed = 0, 0.0, None, None, None
+        if norm is not None:
+            if norm[0] != "dyt":
+                raise KernelError(f"scaled_sum: norm kind {norm[0]!r} (known: 'dyt')")
+            kind, alpha, gain, nbias = 3, float(norm[1]), norm[2], norm[3]
+            self._f32(gain, "scaled_sum norm gain", D)
+            if nbias is not None:
+                self._f32(nbias, "scaled_sum norm bias", D)
+            normed = self.empty(n, D)
+        self._lazy("stream32").tis_scaled_sum(
+            self.code, _ptr(x32), *args, _ptr(chosen.ids if chosen else None), _ptr(chosen.weights if chosen else None),
+            chosen.ids.shape[1] if chosen else 0, chosen.n_experts if chosen else 0, _ptr(chosen.rows if chosen else None),
+            chosen.rows.stride(0) if chosen else 0, _ptr(x32), kind, alpha, _ptr(gain), _ptr(nbias), _ptr(normed),
+            normed.stride(0) if normed is not None else 0, n, D, self._stream())
+        return x32, normed
+
+    _GATED_ACTS = {"gelu_tanh": 0, "silu": 1}
+
+    def gated_act(self, z, hidden: int, act: str, gate_bias=None, up_bias=None, row_scale=None):
+        """act(w * (z[:, :hidden] + gate_bias)) * (w * (z[:, hidden:2 hidden] + up_bias)) in the compute type, w being
+        row_scale [rows] (None: 1). z: [rows, >= 2 hidden] 32-bit (a strided view is fine); act: "gelu_tanh" or "silu"."""
+        n = z.shape[0]
+        self._f32_rows(z, "gated_act z", n, 2 * hidden)
+        for t, what, size in ((gate_bias, "gate bias", hidden), (up_bias, "up bias", hidden), (row_scale, "row factors", n)):
+            if t is not None:
+                self._f32(t, "gated_act " + what, size)
+        if act not in self._GATED_ACTS:
+            raise KernelError(f"gated_act: activation {act!r} (known: {', '.join(self._GATED_ACTS)})")
+        out = self.empty(n, hidden)
+        self._lazy("stream32").tis_gated_act(self.code, _ptr(z), z.stride(0), int(hidden), _ptr(gate_bias), _ptr(up_bias),
+                                             _ptr(row_scale), self._GATED_ACTS[act], _ptr(out), out.stride(0), n,
+                                             self._stream())
+        return out
+
+    def softcap(self, z, cap: float):
+        """z <- cap * tanh(z / cap) on 32-bit rows, in place."""
+        _rows_view(self._check(z, "softcap z", torch.float32), "softcap z")
+        self._lazy("stream32").tis_softcap(_ptr(z), z.stride(0), float(cap), z.shape[0], z.shape[1], self._stream())
+        return z
+
+    # ---- what stands around the scan of a selective state-space mixer ----------------------------------------------
+    def conv_prepare(self, proj, xbc_off, dt_off, taps, tap_bias, dt_bias, neg_a, state, conv_at, batch, n_heads, vdim):
+        """A short causal convolution with silu over `channels` columns of a 32-bit input product (from xbc_off; the
+        first heads * vdim of them are the scan's inputs x), and the step size dt = softplus(proj[:, dt_off + head] +
+        dt_bias) per head. Returns u [rows, channels + heads * vdim + heads] 32-bit: the convolved channels, x * dt,
+        and exp(neg_a * dt). taps: [channels, taps], the last column weighs the row itself. A row's earlier inputs come
+        from the step's rows, and before those from the request's state line (from float conv_at on, [taps - 1]
+        [channels], oldest first)."""
+        n = proj.shape[0]
+        C, K = taps.shape
+        inner = n_heads * vdim
+        self._f32_rows(proj, "conv_prepare projections", n, max(xbc_off + C, dt_off + n_heads))
+        self._f32(taps, "conv taps", C * K)
+        if tap_bias is not None:
+            self._f32(tap_bias, "conv bias", C)
+        self._f32(dt_bias, "dt bias", n_heads)
+        self._f32(neg_a, "decay rates", n_heads)
+        self._check(state, "state", torch.float32)
+        if state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < conv_at + (K - 1) * C:
+            raise KernelError(f"conv_prepare: state {tuple(state.shape)} for {(K - 1) * C} floats from {conv_at}")
+        self._index(batch.row_seq, "row_seq", n)
+        self._index(batch.cu_rows, "cu_rows", batch.n_seqs + 1)
+        self._index(batch.seq_slots, "seq_slots", batch.n_seqs)
+        if max(batch.host_slots, default=0) >= state.shape[0]:
+            raise KernelError(f"conv_prepare: slot {max(batch.host_slots)} of {state.shape[0]}")
+        u = torch.empty(n, C + inner + n_heads, dtype=torch.float32, device=self.device)
+        self._lazy("ssm_parts").tis_conv_prepare(
+            _ptr(proj), proj.stride(0), xbc_off, dt_off, _ptr(taps), _ptr(tap_bias), _ptr(dt_bias), _ptr(neg_a), _ptr(state),
+            state.stride(0), conv_at, _ptr(batch.row_seq), _ptr(batch.cu_rows), _ptr(batch.seq_slots), _ptr(u), u.stride(0),
+            n, C, K, n_heads, vdim, self._stream())
+        return u
+
+    def conv_state_update(self, proj, xbc_off, channels, taps, state, conv_at, batch):
+        """Every request's last taps - 1 convolution inputs (columns xbc_off.. of proj, older ones from the line itself
+        where the step brings fewer rows) into its state line from float conv_at on."""
+        n = proj.shape[0]
+        self._f32_rows(proj, "conv_state_update projections", n, xbc_off + channels)
+        self._check(state, "state", torch.float32)
+        if state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < conv_at + (taps - 1) * channels:
+            raise KernelError(f"conv_state_update: state {tuple(state.shape)} for {(taps - 1) * channels} floats from {conv_at}")
+        self._index(batch.cu_rows, "cu_rows", batch.n_seqs + 1)
+        self._index(batch.seq_slots, "seq_slots", batch.n_seqs)
+        if max(batch.host_slots, default=0) >= state.shape[0]:
+            raise KernelError(f"conv_state_update: slot {max(batch.host_slots)} of {state.shape[0]}")
+        self._lazy("ssm_parts").tis_conv_state_update(_ptr(proj), proj.stride(0), xbc_off, _ptr(state), state.stride(0),
+                                                      conv_at, _ptr(batch.cu_rows), _ptr(batch.seq_slots), batch.n_seqs,
+                                                      channels, taps, self._stream())
+
+    def gated_group_norm(self, y, x, skip, vdim: int, z, gain, eps: float, parts: int):
+        """v = (y + skip[head] * x) * silu(z), each of `parts` equal parts of a row divided by its own root mean square
+        (eps under the root), times gain; in the compute type. y, x, z: [rows, width] 32-bit (strided views are fine);
+        skip [width / vdim] or None (then x is not read); z None: no gate."""
+        n, W = y.shape
+        self._f32_rows(y, "gated_group_norm y", n, W)
+        if skip is not None:
+            self._f32_rows(x, "gated_group_norm x", n, W)
+            if W % vdim:
+                raise KernelError(f"gated_group_norm: width {W} in heads of {vdim}")
+            self._f32(skip, "gated_group_norm skip", W // vdim)
+        if z is not None:
+            self._f32_rows(z, "gated_group_norm z", n, W)
+        self._f32(gain, "gated_group_norm gain", W)
+        if parts < 1 or W % parts:
+            raise KernelError(f"gated_group_norm: width {W} in {parts} parts")
+        out = self.empty(n, W)
+        self._lazy("ssm_parts").tis_gated_group_norm(
+            self.code, _ptr(y), y.stride(0), _ptr(x if skip is not None else None), x.stride(0) if skip is not None else 0,
+            _ptr(skip), int(vdim), _ptr(z), z.stride(0) if z is not None else 0, _ptr(gain), float(eps), _ptr(out),
+            out.stride(0), n, W, int(parts), self._stream())
+        return out
+
     # ---- products in groups: experts, heads -----------------------------------------------------------------
     def _grouped(self, a, lda, a_group, a_div, w, c, ldc, c_group, lists, counts, line, most_rows, act=0):
         G, N, K = w.shape
@@ -1295,17 +1463,20 @@ class HipOps:
             self._grouped(x, x.stride(0), K, 1, w, out[:, out_offset:], out.stride(0), out_group, None, None, 0, n)
         return out
 
-    def route_topk(self, z, correction, scale: float, top: int):
-        """A router's choice: (ids [rows, top] int32, weights [rows, top] 32-bit). s = softmax(z) over a row's outputs;
-        the `top` outputs with the largest s + correction are chosen; an output's weight is s * scale."""
+    def route_topk(self, z, correction, scale: float, top: int, score: str = "softmax"):
+        """A router's choice: (ids [rows, top] int32, weights [rows, top] 32-bit). s = softmax(z) over a row's outputs
+        (score "sigmoid": sigmoid(z), each output by itself); the `top` outputs with the largest s + correction are
+        chosen; an output's weight is s * scale."""
+        if score not in ("softmax", "sigmoid"):
+            raise KernelError(f"route_topk: score {score!r} (known: 'softmax', 'sigmoid')")
         n, E = z.shape
         self._f32_rows(z, "router outputs", n, E)
         if correction is not None:
             self._f32(correction, "router correction", E)
         ids = torch.empty(n, top, dtype=torch.int32, device=self.device)
         weights = torch.empty(n, top, dtype=torch.float32, device=self.device)
-        self._lazy("experts").tis_route_topk(_ptr(z), z.stride(0), _ptr(correction), float(scale), n, E, int(top), _ptr(ids),
-                                             _ptr(weights), self._stream())
+        self._lazy("experts").tis_route_topk(_ptr(z), z.stride(0), _ptr(correction), float(scale), n, E, int(top),
+                                             1 if score == "sigmoid" else 0, _ptr(ids), _ptr(weights), self._stream())
         return ids, weights
 
     def routed_experts(self, x, ids, weights, w_up, w_down, act: str = "gelu_erf", combine: bool = True):
@@ -1341,6 +1512,32 @@ class HipOps:
                                 n, D, self._stream())
         return out
 
+    def gated_experts(self, x, ids, weights, w_gate_up, w_down, act: str = "silu"):
+        """Gated experts whose router weight scales the expert's input: for every (row, choice) the line
+        w_down[e] . (act(w * g) * (w * u)) with [g | u] = w_gate_up[e] . x, e = ids[row, choice], w = weights[row,
+        choice] (an expert without biases applied to w * x), in 32-bit, not summed: a `ChosenExperts` whose weights are
+        None, for a residual sum that adds a row's lines. x: [rows, width] in the compute type; w_gate_up
+        [experts, 2 hidden, width] (the gate's rows first), w_down [experts, width, hidden]."""
+        _rows_view(self._check(x, "experts x"), "experts x")
+        n, D = x.shape
+        top = ids.shape[1]
+        E, F2 = w_gate_up.shape[0], w_gate_up.shape[1]
+        F = F2 // 2
+        self._index(ids, "expert ids", n * top)
+        self._f32(weights, "expert weights", n * top)
+        if E < 1 or F2 % 2 or tuple(w_gate_up.shape) != (E, 2 * F, D) or tuple(w_down.shape) != (E, D, F):
+            raise KernelError(f"gated_experts: matrices {tuple(w_gate_up.shape)} and {tuple(w_down.shape)} for width {D}")
+        y = torch.empty(n * top, D, dtype=torch.float32, device=self.device)
+        if n:
+            lists = torch.empty(E, n, dtype=torch.int32, device=self.device)
+            counts = torch.empty(E, dtype=torch.int32, device=self.device)
+            self._lazy("experts").tis_expert_lists(_ptr(ids), n * top, E, n, _ptr(lists), _ptr(counts), self._stream())
+            z = torch.empty(n * top, 2 * F, dtype=torch.float32, device=self.device)
+            self._grouped(x, x.stride(0), 0, top, w_gate_up, z, z.stride(0), 0, lists, counts, n, n)
+            hidden = self.gated_act(z, F, act, row_scale=weights.view(-1))
+            self._grouped(hidden, hidden.stride(0), 0, 1, w_down, y, D, 0, lists, counts, n, n)
+        return ChosenExperts(y, ids, None, E, x)
+
     # ---- attention with keys and values of different sizes -----------------------------------------------
     def _check_kv_plane(self, plane, n_kv_heads, key_dim, value_dim, page_size):
         self._check(plane, "cache plane")
@@ -1352,18 +1549,21 @@ class HipOps:
     def attention_prepare(self, proj, q_off, k_off, v_off, positions, write_slots, plane, n_heads, n_kv_heads, key_dim,
                           value_dim, page_size, q_gain=None, k_gain=None, q_factor=None, freqs=None, rot_dims=0, eps=0.0,
                           write_cache=True, value_norm=True, q_bias=None, k_bias=None, v_bias=None, temp_coef=0.0,
-                          temp_every=1):
+                          temp_every=1, whole_norm=False, pair_half=False):
         """From a row's 32-bit projections (queries at column q_off, keys at k_off, values at v_off): queries
         [rows, heads*key_dim] in the compute type; keys and values go into the pages at write_slots. On the way, each
         where its argument is given: biases are added; queries and keys are normed per head (RMS, gain of key_dim
         entries); the first rot_dims channels are rotated in interleaved pairs (angle = position * freqs[pair]);
         queries are multiplied by q_factor[head] and by 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1);
-        values are divided by their root mean square (value_norm)."""
+        values are divided by their root mean square (value_norm). whole_norm: the norms run over all heads of a row's
+        queries (keys) at once, with gains of heads * key_dim (kv_heads * key_dim) entries. pair_half: the rotated pairs
+        are (i, i + rot_dims / 2) instead of (2i, 2i + 1)."""
         n = proj.shape[0]
         need = max(q_off + n_heads * key_dim, k_off + n_kv_heads * key_dim, v_off + n_kv_heads * value_dim)
         self._f32_rows(proj, "attention_prepare projections", n, need)
         self._index(positions, "positions", n)
-        for t, what, size in ((q_gain, "query norm gain", key_dim), (k_gain, "key norm gain", key_dim),
+        for t, what, size in ((q_gain, "query norm gain", n_heads * key_dim if whole_norm else key_dim),
+                              (k_gain, "key norm gain", n_kv_heads * key_dim if whole_norm else key_dim),
                               (q_factor, "query factors", n_heads), (q_bias, "query bias", n_heads * key_dim),
                               (k_bias, "key bias", n_kv_heads * key_dim), (v_bias, "value bias", n_kv_heads * value_dim)):
             if t is not None:
@@ -1379,7 +1579,8 @@ class HipOps:
             _ptr(write_slots if write_cache else None), _ptr(plane if write_cache else None), _ptr(q), q.stride(0),
             _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), _ptr(q_gain), _ptr(k_gain), _ptr(q_factor),
             _ptr(freqs if rot_dims else None), int(rot_dims), float(eps), 1 if value_norm else 0, float(temp_coef),
-            int(temp_every), n, n_heads, n_kv_heads, key_dim, value_dim, page_size, self._stream())
+            int(temp_every), 1 if whole_norm else 0, 1 if pair_half else 0, n, n_heads, n_kv_heads, key_dim, value_dim,
+            page_size, self._stream())
         return q
 
     def latent_prepare(self, proj, q_off, c_off, positions, write_slots, plane, n_heads, dim, rot_dim, rank, page_size,
@@ -1472,9 +1673,10 @@ class HipOps:
         return out
 
     def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
-                           scale=None, sink=False, gate=None):
+                           scale=None, sink=False, gate=None, chunk=0):
         """Attention of the rows in `batch` over pages whose keys have key_dim and whose values value_dim channels:
-        [rows, heads*value_dim]. sink: the softmax's denominator also counts a key of score 0 that has no value.
+        [rows, heads*value_dim]. chunk > 0: a row at position p sees only the keys from p - p % chunk on (its own chunk
+        of positions, counted from position 0). sink: the softmax's denominator also counts a key of score 0 that has no value.
         gate: [rows, heads] 32-bit (a strided view is fine); head h's result is multiplied by sigmoid(gate[:, h])."""
         _rows_view(self._check(q, "q"), "q")
         n = q.shape[0]
@@ -1496,7 +1698,7 @@ class HipOps:
         self._lazy("attention_window").tis_attention_window(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, key_dim, value_dim, page_size,
-            int(window), float(scale if scale is not None else key_dim ** -0.5), 1 if sink else 0, _ptr(gate),
+            int(window), int(chunk), float(scale if scale is not None else key_dim ** -0.5), 1 if sink else 0, _ptr(gate),
             gate.stride(0) if gate is not None else 0, self._stream())
         return out
 
@@ -1509,23 +1711,29 @@ class HipOps:
         return n_heads * dim * vdim + (n_heads * blocks * (dim + 1) if kind == "gated_max" else 0)
 
     def state_scan(self, kind, proj, q_off, k_off, v_off, q_scale, state, batch, n_heads, dim, vdim, decay=None,
-                   i_off=0, f_off=0, bias_i=None, bias_f=None, cap=0.0):
+                   i_off=0, f_off=0, bias_i=None, bias_f=None, cap=0.0, qk_group=1, decay_per_head=False):
         """Walk the step's rows of every request through its matrix state, in order, and return o [rows, heads*vdim]
         in 32-bit. kind "decay": S = diag(decay) S + k v^T, o = S^T q. kind "gated_max": scalar log gates per head
         from the columns i_off, f_off of proj (plus biases, capped by cap * tanh(. / cap)), stabilised by a running
         maximum, o normalised by max(|n . q|, exp(-m)) + 1e-6. state: [slots, floats] 32-bit, a line per request.
 
+        qk_group: that many consecutive heads share one set of query and key columns (proj then holds heads / qk_group
+        of them). decay_per_head: `decay` holds one number per head and row instead of one per key channel.
+
         A step whose longest portion has at least two segments' rows (self.scan_segment, 64) is run in segments side
         by side, with a second pass for the states at the segments' starts and a third for what they add to the
         rows' outputs; shorter portions and single tokens are walked in order by one kernel."""
         n = proj.shape[0]
-        need = max(q_off + n_heads * dim, k_off + n_heads * dim, v_off + n_heads * vdim)
+        if qk_group < 1 or n_heads % qk_group:
+            raise KernelError(f"state_scan: {n_heads} heads in groups of {qk_group}")
+        n_qk = n_heads // qk_group
+        need = max(q_off + n_qk * dim, k_off + n_qk * dim, v_off + n_heads * vdim)
         if kind == "gated_max":
             need = max(need, i_off + n_heads, f_off + n_heads)
             self._f32(bias_i, "input gate bias", n_heads)
             self._f32(bias_f, "forget gate bias", n_heads)
         elif kind == "decay":
-            self._f32_rows(decay, "decays", n, n_heads * dim)
+            self._f32_rows(decay, "decays", n, n_heads if decay_per_head else n_heads * dim)
         else:
             raise KernelError(f"state_scan: unknown kind {kind!r}")
         self._f32_rows(proj, "state_scan projections", n, need)
@@ -1551,7 +1759,8 @@ class HipOps:
             0 if kind == "decay" else 1, _ptr(proj), proj.stride(0), q_off, k_off, v_off, float(q_scale), _ptr(decay),
             decay.stride(0) if decay is not None else 0, i_off, f_off, _ptr(bias_i), _ptr(bias_f), float(cap),
             _ptr(state), state.stride(0), _ptr(batch.cu_rows), _ptr(batch.seq_slots), batch.n_seqs, _ptr(out),
-            out.stride(0), n_heads, dim, vdim, segments, seg_len, n, _ptr(workspace), self._stream())
+            out.stride(0), n_heads, dim, vdim, segments, seg_len, n, _ptr(workspace), int(qk_group),
+            1 if decay_per_head else 0, self._stream())
         return out
 
     # ---- sampling ------------------------------------------------------------------------------------

@@ -3,4 +3,4 @@ block arrangements and stage inputs. Importing this package registers the built-
 from .base import (ARRANGEMENTS, FEED_FORWARDS, GATES, MIXERS, NORMS, POSITION_ENCODINGS, STAGE_INPUTS, TOKEN_INPUTS, Arrangement, CallContext,
                    Tensors, build_part, expected_tensors, part_class, to_compute, to_gain)
 from .spec import LayerCall, LayerSpec, ModelSpec, PagedKvNeed, PartSpec, StageSpec, StateNeed
-from . import attention, block, feed_forward, norm, position, prenorm32, recurrent, stage_input, stream32  # noqa: F401  (registration)
+from . import attention, block, feed_forward, norm, parallel32, position, prenorm32, recurrent, stage_input, stream32  # noqa: F401  (registration)

@@ -337,3 +337,83 @@ class LatentAttention:
 
     def forward(self, x, ctx, residual=None):
         return self.ops.linear(self.core(x, ctx), self.w_o, residual=residual)
+
+
+@MIXERS.register("chunked_attention")
+class ChunkedAttention:
+    """Grouped-query softmax attention inside chunks of positions, with biased projections and keys and values of
+    different sizes.
+
+    q = x.Wq^T + bq, k = x.Wk^T + bk, v = x.Wv^T + bv. The whole of a row's queries (all heads side by side) is RMS-normed
+    at once with a gain of heads * key_dim entries, and so is the whole of its keys, before rotation. The first rot_dims
+    channels of every query and key head are rotated in the pairs (i, i + rot_dims / 2) by position * rot_base^(-2i /
+    rot_dims) / rot_factor; the other channels pass. score = q.k * scale. The row at position p sees the keys j <= p
+    with floor(j / chunk) = floor(p / chunk), chunks being counted from position 0 of the sequence (chunk 0: all j <= p).
+    out = softmax-weighted values of all heads . Wo^T + bo. Norms, angles, scores and the softmax are 32-bit.
+
+    params: width, n_heads, n_kv_heads, key_dim, value_dim, scale, eps, rot_dims, rot_base, rot_factor, chunk. tensors,
+    stored [out, in]: q (heads*key_dim, width), k (kv_heads*key_dim, width), v (kv_heads*value_dim, width), q_bias,
+    k_bias, v_bias, q_norm (heads*key_dim,), k_norm (kv_heads*key_dim,), o (width, heads*value_dim), o_bias (width,).
+    """
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, H, G, kd, vd = (params[k] for k in ("width", "n_heads", "n_kv_heads", "key_dim", "value_dim"))
+        return {"q": (H * kd, w), "k": (G * kd, w), "v": (G * vd, w), "q_bias": (H * kd,), "k_bias": (G * kd,),
+                "v_bias": (G * vd,), "q_norm": (H * kd,), "k_norm": (G * kd,), "o": (w, H * vd), "o_bias": (w,)}
+
+    @classmethod
+    def cache_need(cls, params):
+        # every key is kept: a chunk's keys are found through the same block table as any others
+        return PagedKvNeed(params["n_kv_heads"], params["key_dim"], 0, value_dim=params["value_dim"])
+
+    def __init__(self, spec, tensors, ops):
+        from .base import to_gain
+        p = spec.params
+        self.ops = ops
+        self.H, self.G, self.kd, self.vd = int(p["n_heads"]), int(p["n_kv_heads"]), int(p["key_dim"]), int(p["value_dim"])
+        if self.H % self.G:
+            raise ValueError(f"{self.H} query heads are not a multiple of {self.G} key/value heads")
+        self.scale, self.eps, self.chunk = float(p["scale"]), float(p["eps"]), int(p.get("chunk", 0))
+        self.rot_dims = int(p.get("rot_dims", 0))
+        if self.rot_dims % 2 or self.rot_dims > self.kd or self.chunk < 0:
+            raise ValueError(f"{self.rot_dims} rotated channels of a head of {self.kd} (an even number, at most the head), "
+                             f"chunks of {self.chunk}")
+        factor = float(p.get("rot_factor", 1.0))
+        i = torch.arange(self.rot_dims // 2, dtype=torch.float64)
+        freqs = float(p.get("rot_base", 10000.0)) ** (-2.0 * i / max(1, self.rot_dims)) / factor
+        self.freqs = freqs.to(torch.float32).to(ops.device)
+        mats = [tensors.of(spec, k) for k in ("q", "k", "v")]
+        self.k_at = mats[0].shape[0]
+        self.v_at = self.k_at + mats[1].shape[0]
+        self.w_in = to_compute(ops, torch.cat(mats, dim=0))
+        self.q_bias, self.k_bias, self.v_bias, self.o_bias = (to_gain(ops, tensors.of(spec, k))
+                                                              for k in ("q_bias", "k_bias", "v_bias", "o_bias"))
+        self.q_gain, self.k_gain = to_gain(ops, tensors.of(spec, "q_norm")), to_gain(ops, tensors.of(spec, "k_norm"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+
+    def core(self, x, ctx):
+        ops, b = self.ops, ctx.batch
+        proj = ops.linear(x, self.w_in, out_dtype=torch.float32)
+        q = ops.attention_prepare(proj, 0, self.k_at, self.v_at, b.positions, b.write_slots[ctx.group], ctx.plane, self.H,
+                                  self.G, self.kd, self.vd, ctx.page_size, q_gain=self.q_gain, k_gain=self.k_gain,
+                                  freqs=self.freqs, rot_dims=self.rot_dims, eps=self.eps, write_cache=ctx.writes_cache,
+                                  value_norm=False, q_bias=self.q_bias, k_bias=self.k_bias, v_bias=self.v_bias,
+                                  whole_norm=True, pair_half=True)
+        return ops.paged_attention_kv(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, self.vd, ctx.page_size, 0,
+                                      self.scale, chunk=self.chunk)
+
+    def forward_parts(self, x, ctx):
+        """(the result without its output bias, 32-bit; the bias): for a block whose sum adds the bias."""
+        return self.ops.linear(self.core(x, ctx), self.w_o, out_dtype=torch.float32), self.o_bias
+
+    def forward32(self, x, ctx):
+        y, bias = self.forward_parts(x, ctx)
+        return y + bias
+
+    def forward(self, x, ctx, residual=None):
+        y = self.forward32(x, ctx)
+        if residual is not None:
+            y = y + residual.to(torch.float32)
+        return y.to(self.ops.dtype)

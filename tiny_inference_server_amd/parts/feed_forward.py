@@ -91,3 +91,98 @@ class RoutedExperts:
         if residual is not None:
             y = y + residual.to(torch.float32)
         return y.to(self.ops.dtype)
+
+
+@FEED_FORWARDS.register("gated_dense_biased")
+class GatedDenseBiased:
+    """y = Wd . (act(Wg . h + bg) * (Wu . h + bu)) + bd. params: width, hidden, act ("gelu_tanh" or "silu"). tensors,
+    stored [out, in]: gate, up (hidden, width), down (width, hidden), gate_bias, up_bias (hidden,), down_bias (width,)."""
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        d, f = params["width"], params["hidden"]
+        return {"gate": (f, d), "up": (f, d), "down": (d, f), "gate_bias": (f,), "up_bias": (f,), "down_bias": (d,)}
+
+    def __init__(self, spec, tensors, ops):
+        from .base import to_gain
+        self.ops = ops
+        self.act = str(spec.params.get("act", "gelu_tanh"))
+        self.hidden = int(spec.params["hidden"])
+        # one product for both: the gate's rows, then the other factor's
+        self.w_gate_up = to_compute(ops, torch.cat((tensors.of(spec, "gate"), tensors.of(spec, "up")), dim=0))
+        self.w_down = to_compute(ops, tensors.of(spec, "down"))
+        self.gate_bias, self.up_bias, self.down_bias = (to_gain(ops, tensors.of(spec, k))
+                                                        for k in ("gate_bias", "up_bias", "down_bias"))
+
+    def forward_parts(self, rows):
+        """(the result without its output bias, 32-bit; the bias): for a block whose sum adds the bias."""
+        ops = self.ops
+        z = ops.linear(rows, self.w_gate_up, out_dtype=torch.float32)
+        hidden = ops.gated_act(z, self.hidden, self.act, gate_bias=self.gate_bias, up_bias=self.up_bias)
+        return ops.linear(hidden, self.w_down, out_dtype=torch.float32), self.down_bias
+
+    def forward32(self, rows):
+        y, bias = self.forward_parts(rows)
+        return y + bias
+
+    def forward(self, x, residual=None):
+        y = self.forward32(x)
+        if residual is not None:
+            y = y + residual.to(torch.float32)
+        return y.to(self.ops.dtype)
+
+
+@FEED_FORWARDS.register("input_weighted_experts")
+class InputWeightedExperts:
+    """A mixture of gated experts in which a chosen expert's weight multiplies what the expert reads, not its result.
+
+    z = Wr . h (32-bit), s = sigmoid(z) (score "sigmoid") or softmax(z); the `top` experts with the largest s are chosen;
+    a chosen expert's weight is its s, not renormalised; y = sum over the chosen of expert_e(s_e * h) with
+    expert(v) = Wd . (act(Wg . v) * (Wu . v)), no biases. Without biases Wg . (s h) = s (Wg . h), so the weight is
+    applied to the first product's 32-bit results instead of to a rounded copy of the row.
+
+    params: width, hidden, n_experts, top, score, act. tensors, stored [out, in]: router (n_experts, width),
+    gate<e>, up<e> (hidden, width), down<e> (width, hidden).
+    """
+    graph_safe = True
+    sums_in_residual = True     # forward_parts leaves the sum over a row's choices to the block's sum
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, f, E = params["width"], params["hidden"], params["n_experts"]
+        shapes = {"router": (E, w)}
+        for e in range(E):
+            shapes[f"gate{e}"] = (f, w)
+            shapes[f"up{e}"] = (f, w)
+            shapes[f"down{e}"] = (w, f)
+        return shapes
+
+    def __init__(self, spec, tensors, ops):
+        p = spec.params
+        self.ops = ops
+        self.E, self.top = int(p["n_experts"]), int(p["top"])
+        if not 1 <= self.top <= self.E:
+            raise ValueError(f"{self.top} of {self.E} experts")
+        self.score, self.act = str(p.get("score", "sigmoid")), str(p.get("act", "silu"))
+        self.w_router = to_compute(ops, tensors.of(spec, "router"))
+        self.w_gate_up = to_compute(ops, torch.stack([torch.cat((tensors.of(spec, f"gate{e}"), tensors.of(spec, f"up{e}")), dim=0)
+                                                      for e in range(self.E)]))
+        self.w_down = to_compute(ops, torch.stack([tensors.of(spec, f"down{e}") for e in range(self.E)]))
+
+    def forward_parts(self, x):
+        """(the experts' results line by (row, choice), for a sum that adds a row's lines; no bias)."""
+        ops = self.ops
+        z = ops.linear(x, self.w_router, out_dtype=torch.float32)
+        ids, weights = ops.route_topk(z, None, 1.0, self.top, score=self.score)
+        return ops.gated_experts(x, ids, weights, self.w_gate_up, self.w_down, self.act), None
+
+    def forward32(self, x):
+        chosen, _ = self.forward_parts(x)
+        return chosen.results.view(x.shape[0], self.top, -1).sum(1)
+
+    def forward(self, x, residual=None):
+        y = self.forward32(x)
+        if residual is not None:
+            y = y + residual.to(torch.float32)
+        return y.to(self.ops.dtype)

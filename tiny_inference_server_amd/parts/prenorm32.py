@@ -95,9 +95,14 @@ class PreNormStream32(Arrangement):
         if (self.ffn is None) != (self.norm_f is None):
             raise ValueError("a prenorm_stream32 block has a feed-forward and its norm, or neither")
 
+    @staticmethod
+    def _fusable(norm):
+        """Whether the residual sum's kernel can apply this norm (a layer norm or an RMS norm that offers its constants)."""
+        return norm is not None and hasattr(norm, "fused") and norm.fused()[0] in ("layer", "rms")
+
     def _sum(self, x32, y, norm=None, copy=False, y_rms=None):
         """x32 + y with the norm that follows; a norm that cannot be fused is applied on its own."""
-        fused = norm.fused() if norm is not None and hasattr(norm, "fused") else None
+        fused = norm.fused() if self._fusable(norm) else None
         x32, cp, normed = self.ops.residual_norm(x32, y, y_rms=y_rms, copy=copy, norm=fused)
         if norm is not None and fused is None:
             normed = norm(x32)
@@ -111,7 +116,7 @@ class PreNormStream32(Arrangement):
             # (a routed feed-forward leaves the sum over a row's chosen experts to the residual sum's kernel)
             y = self.ffn.forward32(h, combine=False) if getattr(self.ffn, "sums_in_residual", False) else self.ffn.forward32(h)
         # the block's last sum also applies the norm that reads its result next, where that norm can be fused
-        after = ctx.next_norm if hasattr(ctx.next_norm, "fused") else None
+        after = ctx.next_norm if self._fusable(ctx.next_norm) else None
         if self.side is None:
             x32, _, normed = self._sum(x32, y, norm=after)
         else:

@@ -166,3 +166,78 @@ class LightningAttention(_MatrixStateMixer):
         if self._w_in is None:
             self._w_in = to_compute(self.ops, self.input_rows)
         return self.forward_projected(self.ops.linear(x, self._w_in, out_dtype=torch.float32), ctx)
+
+
+@MIXERS.register("selective_state_space")
+class SelectiveStateSpace:
+    """A selective state-space mixer with a scalar decay per head (state-space duality).
+
+    One input product, laid out [z: inner | x: inner | B: groups*state | C: groups*state | dt: heads] with
+    inner = heads * vdim. x, B and C together pass a causal convolution per channel (`taps` taps with a bias, the last
+    tap on the row itself, zeros before the sequence's start) and silu. dt = softplus(dt + dt_bias). Per head h, which
+    reads the B and C of group h // (heads / groups), with the state S of state x vdim numbers:
+    S_t = exp(-exp(a_log[h]) dt_t) S_(t-1) + dt_t B_t x_t^T,  y_t = S_t^T C_t + skip[h] x_t. The heads side by side are
+    multiplied by silu(z), then RMS-normed in norm_groups equal parts (each by its own root mean square) with a gain,
+    and projected by Wo. Everything between the convolution and the norm is 32-bit.
+
+    A request's state line holds S [heads, state, vdim] and after it the convolution's last taps - 1 inputs
+    [taps - 1, channels]; it starts at zero.
+
+    params: width, n_heads, vdim, state, groups, taps, norm_groups, eps. tensors: in (2 inner + 2 groups*state + heads,
+    width) and o (width, inner), stored [out, in]; conv (inner + 2 groups*state, taps), conv_bias, dt_bias (heads,),
+    a_log (heads,), skip (heads,), norm (inner,).
+    """
+    graph_safe = True
+
+    @classmethod
+    def _sizes(cls, params):
+        H, P, N, G, K = (int(params[k]) for k in ("n_heads", "vdim", "state", "groups", "taps"))
+        return H, P, N, G, K, H * P, H * P + 2 * G * N
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        H, P, N, G, K, inner, C = cls._sizes(params)
+        w = params["width"]
+        return {"in": (inner + C + H, w), "conv": (C, K), "conv_bias": (C,), "dt_bias": (H,), "a_log": (H,), "skip": (H,),
+                "norm": (inner,), "o": (w, inner)}
+
+    @classmethod
+    def cache_need(cls, params):
+        H, P, N, G, K, inner, C = cls._sizes(params)
+        return StateNeed((state_floats("decay", H, N, P) + (K - 1) * C,), "float32")
+
+    def __init__(self, spec, tensors, ops):
+        p = spec.params
+        self.ops = ops
+        self.H, self.P, self.N, self.G, self.K, self.inner, self.C = self._sizes(p)
+        self.parts, self.eps = int(p.get("norm_groups", 1)), float(p["eps"])
+        if self.H % self.G or self.inner % self.parts:
+            raise ValueError(f"{self.H} heads over {self.G} groups, a norm of {self.inner} channels in {self.parts} parts")
+        self.w_in = to_compute(ops, tensors.of(spec, "in"))
+        self.taps = to_gain(ops, tensors.of(spec, "conv"))
+        self.tap_bias = to_gain(ops, tensors.of(spec, "conv_bias"))
+        self.dt_bias = to_gain(ops, tensors.of(spec, "dt_bias"))
+        self.neg_a = -torch.exp(to_gain(ops, tensors.of(spec, "a_log")))          # the decay's rate per head, 32-bit
+        self.skip = to_gain(ops, tensors.of(spec, "skip"))
+        self.norm_gain = to_gain(ops, tensors.of(spec, "norm"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+        self.conv_at = state_floats("decay", self.H, self.N, self.P)              # where the line's convolution inputs start
+
+    def core(self, proj, ctx):
+        ops, b = self.ops, ctx.batch
+        H, P, N, G, inner, C = self.H, self.P, self.N, self.G, self.inner, self.C
+        u = ops.conv_prepare(proj, inner, inner + C, self.taps, self.tap_bias, self.dt_bias, self.neg_a, ctx.state,
+                             self.conv_at, b, H, P)
+        ops.conv_state_update(proj, inner, C, self.K, ctx.state, self.conv_at, b)      # after the rows have read the line
+        # the scan's keys are B, its queries C, its values x * dt, its decay exp(-exp(a_log) dt), one per head and row
+        y = ops.state_scan("decay", u, inner + G * N, inner, C, 1.0, ctx.state, b, H, N, P, decay=u[:, C + inner:],
+                           qk_group=H // G, decay_per_head=True)
+        return ops.gated_group_norm(y, u[:, :inner], self.skip, P, proj[:, :inner], self.norm_gain, self.eps, self.parts)
+
+    def forward32(self, x, ctx):
+        proj = self.ops.linear(x, self.w_in, out_dtype=torch.float32)
+        return self.ops.linear(self.core(proj, ctx), self.w_o, out_dtype=torch.float32)
+
+    def forward(self, x, ctx, residual=None):
+        proj = self.ops.linear(x, self.w_in, out_dtype=torch.float32)
+        return self.ops.linear(self.core(proj, ctx), self.w_o, residual=residual)

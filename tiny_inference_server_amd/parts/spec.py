@@ -77,6 +77,7 @@ class ModelSpec:
     lm_head: str                      # tensor name of the output table (vocab, d_model); the same name when tied
     eos_token_id: int = -1
     ignorable: Tuple[str, ...] = ()   # glob patterns of derived buffers a file may also hold
+    logit_softcap: float = 0.0        # cap > 0: logits <- cap * tanh(logits / cap)
 
 
 # What a part needs from the cache manager --------------------------------------------------
