@@ -18,7 +18,7 @@ with temperature, top-k, top-p and repetition penalty, finishing, pages given ba
     python bench.py --workload mixed --size 2.1B     64 requests decoding at contexts of 512..8192 while 2,048-token
                                                      portions of further prompts run in the same steps
 
-    python bench.py --workload designs               the Fikevik and Fipuzen designs beside the grouped-query decoder at equal
+    python bench.py --workload designs               the Fikevik, Fipuzen and Rurorax designs beside the grouped-query decoder at equal
                                                      sizes: prefill and decode throughput of each at a few layer sizes
 
 Each prints one line of the same form; `value` is generated tokens a second over the whole run (serve) or over the
@@ -322,6 +322,22 @@ def fipuzen_config(width, heads, kv_heads, ff, layers, vocab, experts=8, top=2):
                              "token_side": {"dim": 64}, "layers": [kinds[i % 3] for i in range(layers)]})
 
 
+def rurorax_config(width, heads, kv_heads, ff, layers, vocab, experts=8, top=2, chunk=1024):
+    """Chunked attention and a selective state-space mixer in turn (the latter with 2 width / 64 heads of 64 channels and
+    a state of 128 per channel), the feed-forward in turn dense and a mixture of `experts` gated experts of which a row
+    takes `top`, each ff / top wide."""
+    from tiny_inference_server_amd.config import config_from_dict
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": experts, "top": top}}
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": chunk},
+           "rot": {"dims": 64, "base": 1000000.0, "scaling": {"factor": 4.0}}}
+    ssm = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 2, "conv": 4, "norm_groups": 2}
+    kinds = [("attention", att, dense), ("mamba2", ssm, moe), ("attention", att, moe), ("mamba2", ssm, dense)]
+    return config_from_dict({"architecture": "Rurorax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+                             "logit_softcap": 30.0,
+                             "layers": [{"type": t, "mixer": m, "mlp": f} for t, m, f in (kinds[i % 4] for i in range(layers))]})
+
+
 def design_comparison(a, say):
     """Prefill (a.prefill_tokens tokens, one prompt) and decode (batch a.batch, context a.context) of the Fikevik and
     Fipuzen designs and of the grouped-query decoder without prediction heads at the sizes of DESIGN_SIZES, random
@@ -342,6 +358,7 @@ def design_comparison(a, say):
         designs = {
             "fikevik": fikevik_config(width, heads, kv_heads, ff, layers, vocab),
             "fipuzen": fipuzen_config(width, heads, kv_heads, ff, layers, vocab),
+            "rurorax": rurorax_config(width, heads, kv_heads, ff, layers, vocab),
             "gqa": GqaMtpConfig(d_model=width, vocab_size=vocab, max_context=max(8192, a.context), rope_base=500000.0,
                                 n_heads=heads, n_layers=layers, ffn_hidden=ff, group_size=heads // kv_heads, mtp_heads=0,
                                 rms_eps=1e-5, tie_embeddings=False),
@@ -400,7 +417,7 @@ def design_comparison(a, say):
             "warmup": a.warmup, "ms_per_step": points[first].get("decode_ms"), "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": dkey,
             "data": "synthetic: random weights N(0,0.02), uniform random token ids",
-            "config": {"model": "Fikevik and Fipuzen beside GqaMtpTransformer", "sizes": [list(s) for s in DESIGN_SIZES],
+            "config": {"model": "Fikevik, Fipuzen and Rurorax beside GqaMtpTransformer", "sizes": [list(s) for s in DESIGN_SIZES],
                        "global_batch": a.batch, "seq_len": a.context, "prefill_tokens": a.prefill_tokens,
                        "parallelism": "single-gpu"},
             "points": points}
@@ -428,7 +445,7 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", choices=["decode", "serve", "mixed", "designs"], default="decode")
     ap.add_argument("--requests", type=int, default=64, help="serve, mixed: requests (decoding at once)")
-    ap.add_argument("--designs", default="", help="designs: which of fikevik,fipuzen,gqa to run (default: all)")
+    ap.add_argument("--designs", default="", help="designs: which of fikevik,fipuzen,rurorax,gqa to run (default: all)")
     ap.add_argument("--design-sizes", default="", help="designs: which sizes to run, e.g. w2048 (default: all)")
     ap.add_argument("--phase", choices=["both", "prefill", "decode"], default="both", help="designs: what to measure")
     ap.add_argument("--new-tokens", type=int, default=256, help="serve: tokens generated per request")

@@ -144,10 +144,15 @@ def dense_ff(h, t, pre):
     return (gelu_tanh(g) * u) @ w64(t, pre + "down").T + w64(t, pre + "down.b")
 
 
-def route(h, t, pre, top):
-    """(ids [T, top], weights [T, top]): the experts with the largest sigmoid scores, and those scores."""
-    s = torch.sigmoid(h @ w64(t, pre + "router").T)
+def route(h, t, pre, top, margins=None):
+    """(ids [T, top], weights [T, top]): the experts with the largest sigmoid scores, and those scores. margins: a list
+    that receives, per row, how far the last chosen logit lies above the first one left out."""
+    z = h @ w64(t, pre + "router").T
+    s = torch.sigmoid(z)
     w, ids = torch.topk(s, top, dim=-1)
+    if margins is not None and top < z.shape[-1]:
+        ranked = torch.sort(z, dim=-1, descending=True).values
+        margins.extend((ranked[:, top - 1] - ranked[:, top]).tolist())
     return ids, w
 
 
@@ -155,9 +160,9 @@ def expert_ff(h, t, pre):
     return (silu(h @ w64(t, pre + "gate").T) * (h @ w64(t, pre + "up").T)) @ w64(t, pre + "down").T
 
 
-def moe_ff(h, t, pre, mlp, choose=None):
+def moe_ff(h, t, pre, mlp, choose=None, margins=None):
     """sum over a row's chosen experts of expert(weight * h). choose(h) -> (ids, weights) replaces the router's choice."""
-    ids, w = choose(h) if choose is not None else route(h, t, pre, mlp["router"]["top"])
+    ids, w = choose(h) if choose is not None else route(h, t, pre, mlp["router"]["top"], margins)
     y = torch.zeros_like(h)
     for r in range(h.shape[0]):
         for e, we in zip(ids[r].tolist(), w[r]):
@@ -169,7 +174,7 @@ def norm_of(x, t, name):
     return dynamic_tanh(x, w64(t, name + ".alpha"), w64(t, name), w64(t, name + ".b"))
 
 
-def layer(x, t, i, entry, eps, choose=None):
+def layer(x, t, i, entry, eps, choose=None, margins=None):
     pre = f"l{i}."
     h = norm_of(x, t, pre + "norm1")
     if entry["type"] == "attention":
@@ -181,19 +186,28 @@ def layer(x, t, i, entry, eps, choose=None):
     out = x + y * w64(t, pre + "ls1")
     mlp = entry.get("mlp")
     if mlp is not None:
-        f = dense_ff(h, t, pre + "mlp.") if mlp["kind"] == "dense" else moe_ff(h, t, pre + "mlp.", mlp, choose)
+        f = dense_ff(h, t, pre + "mlp.") if mlp["kind"] == "dense" else moe_ff(h, t, pre + "mlp.", mlp, choose, margins)
         out = out + f * w64(t, pre + "ls2")
     return out
 
 
-def forward(config, tensors, tokens, streams=None, choose=None):
-    """Logits [T, vocab] in float64. streams: a list that receives the stream after every layer."""
+def forward(config, tensors, tokens, streams=None, choose=None, margins=None):
+    """Logits [T, vocab] in float64. streams: a list that receives the stream after every layer. margins: a list that
+    receives every routed row's margin (see route)."""
     eps = config["norm"]["eps"]
     x = w64(tensors, "embed")[torch.as_tensor(tokens, dtype=torch.long)]
     for i, entry in enumerate(config["layers"]):
-        x = layer(x, tensors, i, entry, eps, choose)
+        x = layer(x, tensors, i, entry, eps, choose, margins)
         if streams is not None:
             streams.append(x.clone())
     logits = norm_of(x, tensors, "final.norm") @ w64(tensors, "embed").T
     cap = config.get("logit_softcap")
     return cap * torch.tanh(logits / cap) if cap else logits
+
+
+def greedy_generate(config, tensors, prompt, n_new):
+    """n_new tokens, each the largest logit of the whole sequence so far run again from its start."""
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(forward(config, tensors, ids)[-1].argmax()))
+    return ids[len(prompt):]

@@ -136,7 +136,7 @@ def make_paged(kv_lens, n_kv, hd, page_size, dtype, seed, shuffle=True):
 def dense_reference(q, k, v, group, pos, window=0):
     """One row: query heads [NH, hd] against keys [0, pos] by library attention on repeated kv heads
     (the reference's own oracle: test_gqa_paged.py:39-44)."""
-    lo = max(0, pos - window + 1) if window else 0
+    lo = max(0, pos - window + 1) if window > 0 else pos - pos % (-window) if window < 0 else 0     # < 0: chunks of -window
     kq = k[lo:pos + 1].double().repeat_interleave(group, dim=1).transpose(0, 1)     # [NH, keys, hd]
     vq = v[lo:pos + 1].double().repeat_interleave(group, dim=1).transpose(0, 1)
     return torch.nn.functional.scaled_dot_product_attention(q.double()[:, None, :], kq, vq)[:, 0, :]
@@ -181,7 +181,7 @@ def test_paged_attention_single_rows(ops_for, dtype, n_heads, n_kv, hd, page_siz
         assert not torch.allclose(got[0].view(n_heads, hd).double(), bad, rtol=2e-2, atol=2e-2)
 
 
-@pytest.mark.parametrize("window", [1000, 500])
+@pytest.mark.parametrize("window", [1000, 500, -600])
 def test_single_rows_of_uneven_lengths_behind_a_window(ops_for, window):
     """Decoded tokens of requests that differ widely in length, in a layer that sees a window ending inside a page:
     the splits are planned from what each row sees (the window's keys), not from its request's length."""
@@ -194,7 +194,7 @@ def test_single_rows_of_uneven_lengths_behind_a_window(ops_for, window):
     entries, _ = hip_ops.decode_items(seq_rows, n_heads, n_kv, hd, window=window)
     live = entries[entries[:, 0] >= 0]
     for i, L in enumerate(kv_lens):          # no row gets more splits than its window has steps of 32 keys
-        steps = (L + 31 - (max(0, L - window) & ~31)) // 32
+        steps = (L + 31 - (hip_ops.first_key(L - 1, window) & ~31)) // 32
         assert 1 <= (live[live[:, 0] == i][:, 1] >> 16).max() <= steps
     plane, tables, ks, vs = make_paged(kv_lens, n_kv, hd, page_size, torch.bfloat16, seed=27)
     B = len(kv_lens)
@@ -297,7 +297,7 @@ def test_paged_attention_portions_and_window(ops_for, dtype, n_heads, n_kv, hd, 
                             block_tables={"g": tables.cuda()}, max_kv_len=max(kv_lens), extras={},
                             n_rows=R, max_seq_rows=200, seq_rows=seq_rows)
     t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
-    for window in (0, 37):
+    for window in (0, 37, -37, -120):       # all keys, the last 37, chunks of 37 and of 120 positions
         got = ops.paged_attention(q.cuda(), plane.cuda(), batch, "g", n_heads, n_kv, hd, window=window).cpu()
         for r in range(0, R, 7):
             want = dense_reference(q[r].view(n_heads, hd), ks[row_seq[r]], vs[row_seq[r]], group, positions[r], window)
@@ -334,7 +334,8 @@ def test_mixed_rows_with_key_splits_chosen_item_by_item(ops_for, n_heads, n_kv, 
 
 @pytest.mark.parametrize("n_heads,n_kv,hd,page_size,window", [
     (12, 3, 128, 16, 0), (12, 3, 128, 16, 100), (4, 4, 64, 16, 0), (6, 2, 48, 32, 0), (16, 2, 32, 48, 45),
-    (2, 1, 256, 16, 0), (5, 1, 16, 16, 33), (20, 1, 32, 16, 0)])
+    (2, 1, 256, 16, 0), (5, 1, 16, 16, 33), (20, 1, 32, 16, 0), (12, 3, 128, 16, -100), (4, 2, 64, 32, -333),
+    (6, 2, 48, 16, -64)])
 @pytest.mark.parametrize("splits", [False, True])
 def test_long_portions_by_tiles(ops_for, monkeypatch, n_heads, n_kv, hd, page_size, window, splits):
     """Portions long enough for the workgroup kernel (tiles of rows whose four waves share each step's keys through
@@ -390,6 +391,9 @@ def test_paged_attention_of_drawn_batches(ops_for, monkeypatch, first):
         hd = rng.choice([16, 32, 48, 64, 80, 96, 128, 128, 160, 256])
         page = rng.choice([16, 16, 32, 48, 64])
         window = rng.choice([0, 0, 0, rng.randint(5, 900)])
+        chunks = random.Random(case + 5000)         # (a draw of its own: the other draws stay what they were)
+        if chunks.random() < 0.3:
+            window = -chunks.choice([chunks.randint(1, 900), 32, 64, 200, 1])       # chunks of that many positions
         n_heads = n_kv * group
         n_req = rng.randint(1, 4) if rng.random() < 0.8 else rng.randint(10, 24)
         segs = []

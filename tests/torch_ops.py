@@ -132,7 +132,8 @@ class TorchOps:
         seq = batch.row_seq.tolist()
         for r in range(n):
             p = pos[r]
-            first = max(0, p - window + 1) if window > 0 else 0
+            # window > 0: the last `window` keys; window < 0: the row's own chunk of -window positions; 0: all
+            first = max(0, p - window + 1) if window > 0 else p - p % (-window) if window < 0 else 0
             js = torch.arange(first, p + 1)
             pages = tables[seq[r]].long()[js // page_size]
             k = plane[pages, 0, :, js % page_size].float()       # [keys, kvh, hd]

@@ -44,6 +44,15 @@ static constexpr int HD = TIS_HD;
 static constexpr int DC = (HD + 31) / 32;   // 32-wide chunks of the head for Q.K
 static constexpr int DB = HD / 16;          // 16-wide blocks of the head for P.V
 
+// The first key that the row at position p sees. window > 0: the last `window` keys; window < 0: the keys of the row's own
+// chunk of -window positions, chunks counted from position 0; 0: all. Never decreases as p grows, which is what the
+// kernels' ranges of steps rest on.
+__device__ __forceinline__ int first_key(int p, int window) {
+  if (window > 0) return p - window + 1 > 0 ? p - window + 1 : 0;
+  if (window < 0) return p > 0 ? p - p % (-window) : 0;
+  return 0;
+}
+
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x4 load4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
 
@@ -117,7 +126,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     col_row[nb] = row0 + (col_ok[nb] ? ro : 0);
     col_head[nb] = kvh * group_size + c % group_size;
     col_pos[nb] = col_ok[nb] ? p_first + ro : -1;
-    col_lo[nb] = (window > 0 && col_pos[nb] - window + 1 > 0) ? col_pos[nb] - window + 1 : 0;
+    col_lo[nb] = first_key(col_pos[nb], window);
   }
 
   // queries: the B operand of S^T, kept in registers for the whole key range
@@ -133,10 +142,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     }
 
   // this wave's share of the item's keys, in steps of 32 from a multiple of 32
-  int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+  int k_lo = first_key(p_first, window);
   k_lo &= ~31;
   const int k_hi = p_last + 1;
-  const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;   // the largest window start
+  const int lo_last = first_key(p_last, window);   // the largest window start
   const int n_steps = (k_hi - k_lo + 31) / 32;
   // The grid offers every item n_splits waves a kv head. With min_steps an item takes only as many of them as
   // leaves each at least that many steps, so that short items are not cut into crumbs while long ones (the last
@@ -230,7 +239,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
       // Values of keys that no column of the item may see (slots past its last position, keys before its window,
       // tiles past its range) are set to zero and not merely weighted by zero: what lies there is whatever an
       // earlier owner of the page left, possibly not even finite.
-      const int lo_first = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+      const int lo_first = first_key(p_first, window);
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -459,7 +468,7 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(HD <= 1
   const int col_row = row0 + (col_ok ? ro : 0);
   const int col_head = kvh * group_size + c32 % group_size;
   const int col_pos = col_ok ? p_first + ro : -1;
-  const int col_lo = (window > 0 && col_pos - window + 1 > 0) ? col_pos - window + 1 : 0;
+  const int col_lo = first_key(col_pos, window);
   bf16x8 qb[KC];
 #pragma unroll
   for (int kc = 0; kc < KC; ++kc) {
@@ -469,7 +478,7 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(HD <= 1
   }
 
   // the tile's keys and this workgroup's share of them, as in the wave kernel
-  const int t_lo = (window > 0 && tp_first - window + 1 > 0) ? tp_first - window + 1 : 0;   // first key any row sees
+  const int t_lo = first_key(tp_first, window);   // first key any row sees
   const int k_lo = t_lo & ~31;
   const int k_hi = tp_last + 1;
   const int n_steps = (k_hi - k_lo + 31) / 32;
@@ -480,8 +489,8 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(HD <= 1
   const int per_split = (n_steps + item_splits - 1) / item_splits;
   const int s_begin = split * per_split;
   const int s_end = min(n_steps, s_begin + per_split);
-  const int w_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;    // first key the wave sees
-  const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+  const int w_lo = first_key(p_first, window);    // first key the wave sees
+  const int lo_last = first_key(p_last, window);
 
   const long page_stride = 2L * n_kv_heads * page_size * HD;
   const long k_head = (long)kvh * page_size * HD;

@@ -302,6 +302,22 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
     return nb, cut(rest, max(1, (16 * nb) // group_size))[0], tiles, steps
 
 
+def first_key(pos: int, window: int) -> int:
+    """The first key that the row at position pos sees, as the matrix-core attention kernels count: window > 0: the
+    last `window` keys; window < 0: the keys of the row's own chunk of -window positions, chunks counted from position
+    0; 0: all."""
+    if window > 0:
+        return max(0, pos - window + 1)
+    if window < 0:
+        return pos - pos % (-window)
+    return 0
+
+
+def row_steps(pos: int, window: int) -> int:
+    """32-key steps that a wave walks for the row at position pos: from a multiple of 32 to the row's own key."""
+    return (pos + 32 - (first_key(pos, window) & ~31)) >> 5
+
+
 def uneven_lengths(seq_rows, window: int = 0) -> bool:
     """Whether a step of single rows holds requests of such different lengths that equal split counts would leave the
     longest request's waves running on alone: then the splits are planned request by request (decode_items). With a
@@ -313,7 +329,7 @@ def uneven_lengths(seq_rows, window: int = 0) -> bool:
     for _, p0, rows in seq_rows:            # (one pass: this runs for every step of decoded tokens)
         if rows != 1:
             return False
-        steps = (p0 + 32) >> 5 if window <= 0 or p0 < window else (p0 + 32 - ((p0 - window + 1) & ~31)) >> 5
+        steps = row_steps(p0, window)
         total += steps
         if steps > longest:
             longest = steps
@@ -355,7 +371,7 @@ def decode_items(seq_rows, n_heads: int, n_kv_heads: int, head_dim: int, workspa
     pos = np.fromiter((p0 for _, p0, _ in seq_rows), dtype=np.int64, count=n)
     # a row at position p sees p + 1 keys, or the last `window` of them; the kernel walks them in steps of 32 from a
     # multiple of 32
-    first = np.maximum(0, pos - window + 1) & ~31 if window > 0 else 0
+    first = np.maximum(0, pos - window + 1) & ~31 if window > 0 else (pos - pos % (-window)) & ~31 if window < 0 else 0
     steps = (pos + 32 - first) // 32
     fewest = max(1, _ATTN_MIN_SPLIT_KEYS // 32)
     even = max(fewest, -(-int(steps.sum()) * n_kv_heads // max(1, int(planned_target_waves(n_kv_heads, units) * share))))
@@ -403,9 +419,8 @@ def planned_beside_tiles(seq_rows, items, tiles, tile_steps, n_heads: int, n_kv_
     if len(singles) != n_items or not uneven_lengths(singles, window):
         return None
     # what the rows take at the rate a step of decoded tokens streams keys and values, against the tiles' estimate
-    row_steps = sum((p0 + 32) >> 5 if window <= 0 or p0 < window else (p0 + 32 - ((p0 - window + 1) & ~31)) >> 5
-                    for _, p0, _ in singles)
-    rows_us = row_steps * n_kv_heads * 64 * head_dim * 2 / _ATTN_DECODE_BYTES_PER_US
+    steps_of_rows = sum(row_steps(p0, window) for _, p0, _ in singles)
+    rows_us = steps_of_rows * n_kv_heads * 64 * head_dim * 2 / _ATTN_DECODE_BYTES_PER_US
     cut, cut_steps = _tiles_cut(all_rows, len(tiles), tile_steps, n_heads, n_kv_heads, head_dim)
     tiles_us = min(_tiles_us(all_rows, len(tiles), tile_steps[0], tile_steps[1], cut, cut_steps, n_heads, n_kv_heads,
                              head_dim, True, units))
@@ -963,6 +978,9 @@ class HipOps:
         the general kernel. sink: the softmax's denominator also counts a key of score 0 that has no value. gate
         ([rows, heads] 32-bit, a strided view is fine): head h's result is multiplied by sigmoid(gate[:, h]). Calls with
         a sink or a gate that the matrix-core kernels do not take go to the kernel for keys and values of any sizes.
+        window > 0: a row sees its last `window` keys; window < 0: the keys of its own chunk of -window positions, chunks
+        counted from position 0 (such calls, too, go to the kernel for any sizes where the matrix-core kernels do not
+        take them); 0: all.
         """
         group_name = group
         if (sink or gate is not None) and slopes is not None:
@@ -1072,9 +1090,11 @@ class HipOps:
             if gate is not None:
                 self.head_gate(out, gate, n_heads, head_dim)
             return out
-        if sink or gate is not None:
+        if sink or gate is not None or window < 0:
+            if slopes is not None:
+                raise KernelError("attention: score slopes do not go with chunks of positions")
             return self.paged_attention_kv(q, plane, batch, group_name, n_heads, n_kv_heads, head_dim, head_dim, page_size,
-                                           window, scale, sink=sink, gate=gate)
+                                           max(0, window), scale, sink=sink, gate=gate, chunk=max(0, -window))
         self.attn_generic.tis_attention_generic(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, head_dim, page_size, int(window),

@@ -392,6 +392,21 @@ class ChunkedAttention:
                                                               for k in ("q_bias", "k_bias", "v_bias", "o_bias"))
         self.q_gain, self.k_gain = to_gain(ops, tensors.of(spec, "q_norm")), to_gain(ops, tensors.of(spec, "k_norm"))
         self.w_o = to_compute(ops, tensors.of(spec, "o"))
+        self.same = self.kd == self.vd        # then the pages have the layout every attention kernel reads
+        self.span = -self.chunk               # how the attention kernels for one size are told of chunks: a negative window
+
+    # the matrix-core kernels' work lists, where keys and values are of one size (see GqaAttention)
+    def plan_key(self):
+        if not self.same or not hasattr(self.ops, "plan_attention"):
+            return None
+        return ("attention", self.H, self.G, self.kd, self.span)
+
+    def plan_mode(self, seq_rows):
+        mode = getattr(self.ops, "plan_attention_mode", None)
+        return mode(seq_rows, self.span) if mode is not None and self.same else None
+
+    def plan_rows(self, seq_rows, add, mode=None):
+        return self.ops.plan_attention(self.H, self.G, self.kd, seq_rows, add, mode, self.span)
 
     def core(self, x, ctx):
         ops, b = self.ops, ctx.batch
@@ -401,6 +416,8 @@ class ChunkedAttention:
                                   freqs=self.freqs, rot_dims=self.rot_dims, eps=self.eps, write_cache=ctx.writes_cache,
                                   value_norm=False, q_bias=self.q_bias, k_bias=self.k_bias, v_bias=self.v_bias,
                                   whole_norm=True, pair_half=True)
+        if self.same:
+            return ops.paged_attention(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, self.span, self.scale)
         return ops.paged_attention_kv(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, self.vd, ctx.page_size, 0,
                                       self.scale, chunk=self.chunk)
 
