@@ -64,12 +64,17 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
       const int n_all = (is_q ? H : G) * KD;
       const float* all = proj + r * ldp + (is_q ? q_off : k_off);
       const float* all_bias = is_q ? a.q_bias : a.k_bias;
-      float ss = 0.f;
-      for (int e = lane; e < n_all; e += TIS_WAVE) {
-        const float v = all[e] + (all_bias ? all_bias[e] : 0.f);
-        ss += v * v;
+      // (four sums side by side, so that a lane's loads are in flight together; the order depends on n_all alone)
+      float part[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int e0 = lane; e0 < n_all; e0 += 4 * TIS_WAVE) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int e = e0 + i * TIS_WAVE;
+          const float v = e < n_all ? all[e] + (all_bias ? all_bias[e] : 0.f) : 0.f;
+          part[i] += v * v;
+        }
       }
-      ss = wave_sum(ss);
+      const float ss = wave_sum((part[0] + part[1]) + (part[2] + part[3]));
       inv = 1.f / sqrtf(ss / (float)n_all + a.eps);
       gain += (long)h * KD;
     } else if (gain) {

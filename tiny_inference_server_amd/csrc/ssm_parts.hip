@@ -21,8 +21,10 @@ static constexpr int SSM_MAX_TAPS = 16;
 __device__ __forceinline__ float ssm_silu(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float ssm_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
-// grid (rows). proj: a row's input product in 32-bit, the convolution's channels from xbc_off, dt_raw from dt_off.
-// u (out) [rows][ldu]: [conv channels (x: H*P, then B and C) | x * dt: H*P | decay: H].
+// grid (rows, blocks of SSM_THREADS channels): a thread has one channel of one row, so that a step of a few rows still
+// fills the chip and no thread walks a chain of dependent loads. proj: a row's input product in 32-bit, the convolution's
+// channels from xbc_off, dt_raw from dt_off. u (out) [rows][ldu]: [conv channels (x: H*P, then B and C) | x * dt: H*P |
+// decay: H].
 __global__ __launch_bounds__(SSM_THREADS) void conv_prepare_kernel(
     const float* __restrict__ proj, long ldp, int xbc_off, int dt_off, const float* __restrict__ taps,
     const float* __restrict__ tap_bias, const float* __restrict__ dt_bias, const float* __restrict__ neg_a,
@@ -35,12 +37,21 @@ __global__ __launch_bounds__(SSM_THREADS) void conv_prepare_kernel(
   const float* old = state + (long)seq_slots[seq] * state_ld + conv_at;
   const float* row = proj + r * ldp;
   const int inner = H * P;
-  for (int c = threadIdx.x; c < C; c += SSM_THREADS) {
-    float acc = tap_bias ? tap_bias[c] : 0.f;
-    for (int j = 0; j < K; ++j) {
+  const int c = blockIdx.y * SSM_THREADS + threadIdx.x;
+  if (c < C) {
+    float v[SSM_MAX_TAPS], w[SSM_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < SSM_MAX_TAPS; ++j) {                // every load first, then the sum in the taps' order
+      if (j >= K) break;
       const int back = K - 1 - j;                           // the last tap weighs the row itself
-      const float v = back <= t ? row[xbc_off + c - (long)back * ldp] : old[(long)(K - 1 + t - back) * C + c];
-      acc += taps[(long)c * K + j] * v;
+      v[j] = back <= t ? row[xbc_off + c - (long)back * ldp] : old[(long)(K - 1 + t - back) * C + c];
+      w[j] = taps[(long)c * K + j];
+    }
+    float acc = tap_bias ? tap_bias[c] : 0.f;
+#pragma unroll
+    for (int j = 0; j < SSM_MAX_TAPS; ++j) {
+      if (j >= K) break;
+      acc += w[j] * v[j];
     }
     const float y = ssm_silu(acc);
     u[r * ldu + c] = y;
@@ -49,39 +60,33 @@ __global__ __launch_bounds__(SSM_THREADS) void conv_prepare_kernel(
       u[r * ldu + C + c] = y * ssm_softplus(row[dt_off + h] + dt_bias[h]);
     }
   }
-  for (int h = threadIdx.x; h < H; h += SSM_THREADS)
-    u[r * ldu + C + inner + h] = expf(neg_a[h] * ssm_softplus(row[dt_off + h] + dt_bias[h]));
+  if (blockIdx.y == 0)
+    for (int h = threadIdx.x; h < H; h += SSM_THREADS)
+      u[r * ldu + C + inner + h] = expf(neg_a[h] * ssm_softplus(row[dt_off + h] + dt_bias[h]));
 }
 
-// grid (requests of the step). Every thread owns channels: it reads a channel's old inputs before it writes the new.
+// grid (requests of the step, blocks of SSM_THREADS channels). A thread owns one channel of one request: it reads the
+// channel's old inputs before it writes the new.
 __global__ __launch_bounds__(SSM_THREADS) void conv_state_update_kernel(const float* __restrict__ proj, long ldp, int xbc_off,
                                                                          float* __restrict__ state, long state_ld,
                                                                          int conv_at, const int* __restrict__ cu_rows,
                                                                          const int* __restrict__ seq_slots, int C, int K) {
   const int seq = blockIdx.x;
   const int r0 = cu_rows[seq], n = cu_rows[seq + 1] - r0;
-  if (n <= 0) return;
+  const int c = blockIdx.y * SSM_THREADS + threadIdx.x;
+  if (n <= 0 || c >= C) return;
   float* line = state + (long)seq_slots[seq] * state_ld + conv_at;
-  for (int c = threadIdx.x; c < C; c += SSM_THREADS) {
-    float keep[SSM_MAX_TAPS];
+  float next[SSM_MAX_TAPS];
 #pragma unroll
-    for (int k = 0; k < SSM_MAX_TAPS; ++k)
-      if (k < K - 1) keep[k] = line[(long)k * C + c];
+  for (int k = 0; k < SSM_MAX_TAPS; ++k) {
+    if (k >= K - 1) break;
+    const int at = n - (K - 1) + k;                         // which row of the step becomes entry k (negative: an old one)
+    next[k] = at >= 0 ? proj[(long)(r0 + at) * ldp + xbc_off + c] : line[(long)(k + n) * C + c];
+  }
 #pragma unroll
-    for (int k = 0; k < SSM_MAX_TAPS; ++k) {
-      if (k >= K - 1) continue;
-      const int at = n - (K - 1) + k;                       // which row of the step becomes entry k (negative: an old one)
-      float v;
-      if (at >= 0) {
-        v = proj[(long)(r0 + at) * ldp + xbc_off + c];
-      } else {
-        v = 0.f;
-#pragma unroll
-        for (int o = 0; o < SSM_MAX_TAPS; ++o)
-          if (o == k + n) v = keep[o];
-      }
-      line[(long)k * C + c] = v;
-    }
+  for (int k = 0; k < SSM_MAX_TAPS; ++k) {
+    if (k >= K - 1) break;
+    line[(long)k * C + c] = next[k];
   }
 }
 
@@ -101,7 +106,27 @@ __global__ __launch_bounds__(SSM_THREADS) void gated_group_norm_kernel(
     if (z) v *= ssm_silu(z[r * ldz + c]);
     return v;
   };
+  // a part of up to SSM_KEEP * SSM_THREADS columns stays in registers between the sum of squares and the division (its
+  // loads are all in flight together); a wider one is read again
+  constexpr int SSM_KEEP = 8;
+  float kept[SSM_KEEP];
   float ss = 0.f;
+  if (part_width <= SSM_KEEP * SSM_THREADS) {
+#pragma unroll
+    for (int i = 0; i < SSM_KEEP; ++i) {
+      const int e = threadIdx.x + i * SSM_THREADS;
+      kept[i] = e < part_width ? value(c0 + e) : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < SSM_KEEP; ++i) ss += kept[i] * kept[i];
+    const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)part_width + eps);
+#pragma unroll
+    for (int i = 0; i < SSM_KEEP; ++i) {
+      const int e = threadIdx.x + i * SSM_THREADS;
+      if (e < part_width) out[r * ldo + c0 + e] = from_f<T>(kept[i] * inv * gain[c0 + e]);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < part_width; e += SSM_THREADS) {
     const float v = value(c0 + e);
     ss += v * v;
@@ -122,8 +147,9 @@ TIS_EXPORT int tis_conv_prepare(const float* proj, long ldp, int xbc_off, int dt
   if (ldu < (long)C + (long)H * P + H || state_ld < (long)conv_at + (long)(K - 1) * C)
     return tis_fail("conv_prepare: rows of %ld floats for %ld, state lines of %ld for %ld", ldu, (long)C + (long)H * P + H,
                     state_ld, (long)conv_at + (long)(K - 1) * C);
-  conv_prepare_kernel<<<rows, SSM_THREADS, 0, stream>>>(proj, ldp, xbc_off, dt_off, taps, tap_bias, dt_bias, neg_a, state,
-                                                        state_ld, conv_at, row_seq, cu_rows, seq_slots, u, ldu, C, K, H, P);
+  conv_prepare_kernel<<<dim3(rows, (C + SSM_THREADS - 1) / SSM_THREADS), SSM_THREADS, 0, stream>>>(
+      proj, ldp, xbc_off, dt_off, taps, tap_bias, dt_bias, neg_a, state, state_ld, conv_at, row_seq, cu_rows, seq_slots, u, ldu,
+      C, K, H, P);
   return tis_launch_status("conv_prepare");
 }
 
@@ -133,7 +159,7 @@ TIS_EXPORT int tis_conv_state_update(const float* proj, long ldp, int xbc_off, f
   if (n_seqs == 0 || K == 1) return 0;
   if (n_seqs < 0 || C < 1 || K < 1 || K > SSM_MAX_TAPS || state_ld < (long)conv_at + (long)(K - 1) * C)
     return tis_fail("conv_state_update: bad size requests=%d channels=%d taps=%d state line=%ld", n_seqs, C, K, state_ld);
-  conv_state_update_kernel<<<n_seqs, SSM_THREADS, 0, stream>>>(proj, ldp, xbc_off, state, state_ld, conv_at, cu_rows,
+  conv_state_update_kernel<<<dim3(n_seqs, (C + SSM_THREADS - 1) / SSM_THREADS), SSM_THREADS, 0, stream>>>(proj, ldp, xbc_off, state, state_ld, conv_at, cu_rows,
                                                                seq_slots, C, K);
   return tis_launch_status("conv_state_update");
 }
