@@ -5,7 +5,7 @@ some, as many as query heads), key and value sizes (equal and different), chunks
 test sequence and none at all, rotated channels (all, some, none) with and without scaled frequencies, state sizes,
 groups (one, some, as many as heads), convolution taps from 1 (no inputs kept) to 4, norm parts, dense and routed
 feed-forwards with top from 1 to all experts, a layer without a feed-forward, a model without a cap on its logits, a
-width that is no multiple of 8.
+width that is no multiple of 8, and sizes of one wherever a size may be one.
 
 Routing and bfloat16: an expert is chosen by comparing scores, and a bfloat16 engine may turn a close comparison the
 other way; the plain implementation would then describe another model. So the engine's bfloat16 tests run the
@@ -68,7 +68,7 @@ def _configs():
                          dense(attention(2, 2, 32, 32, 0.15, chunk=7), 0),
                          dense(ssm(3, 16, 8, 1, 2), 56)], cap=9.0)
     # a width that is no multiple of 8, no cap, chunks of one position (a row sees itself alone), every channel rotated
-    # with unscaled frequencies, as many groups as heads would have been 1 head a group: here 2; all experts chosen
+    # with unscaled frequencies, two heads a group, all experts chosen, a norm in three parts
     B = config(44, 97, [moe(ssm(6, 4, 5, 3, 3, parts=3), 20, 3, 3),
                         dense(attention(6, 1, 8, 8, 0.3, chunk=1, dims=8, base=50.0), 28),
                         moe(attention(3, 3, 12, 4, 0.25, chunk=33, dims=4, base=300.0, factor=1.5), 12, 5, 1)], eps=1e-6)
@@ -86,7 +86,11 @@ def _configs():
     E = config(56, 150, [moe(attention(3, 3, 20, 36, 0.22, dims=None), 24, 7, 3),
                          dense(attention(2, 1, 40, 16, 0.16, chunk=4096, dims=10, base=1e4, factor=8.0), 48),
                          dense(attention(4, 2, 8, 8, 0.35, chunk=16, dims=2), 0)])
-    return {"A": A, "B": B, "C": C, "D": D, "E": E}
+    # ones wherever a size may be one: a single head, one key/value head, one group, a state of one number per value
+    # channel, values of one channel, one expert, one norm part per channel, chunks longer than a page and a single tap
+    F = config(24, 61, [moe(ssm(1, 8, 1, 1, 2), 8, 1, 1), dense(attention(1, 1, 8, 8, 0.4, chunk=19, dims=8, base=100.0), 16),
+                        dense(ssm(3, 1, 6, 1, 1, parts=3), 0), moe(attention(2, 1, 6, 1, 0.5, chunk=2), 4, 2, 1)], cap=3.0)
+    return {"A": A, "B": B, "C": C, "D": D, "E": E, "F": F}
 
 
 CONFIGS = _configs()

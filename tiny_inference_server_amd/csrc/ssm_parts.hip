@@ -21,8 +21,9 @@ static constexpr int SSM_MAX_TAPS = 16;
 __device__ __forceinline__ float ssm_silu(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float ssm_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
-// grid (rows, blocks of SSM_THREADS channels): a thread has one channel of one row, so that a step of a few rows still
-// fills the chip and no thread walks a chain of dependent loads. proj: a row's input product in 32-bit, the convolution's
+// grid (rows * blocks of SSM_THREADS * per_thread channels, a row's blocks side by side): with few rows a thread has one
+// channel of one row (per_thread 1), so that the step still fills the chip and no thread walks a chain of dependent
+// loads; with many rows it has several, so that the grid is not made of crumbs. proj: a row's input product in 32-bit, the convolution's
 // channels from xbc_off, dt_raw from dt_off. u (out) [rows][ldu]: [conv channels (x: H*P, then B and C) | x * dt: H*P |
 // decay: H].
 __global__ __launch_bounds__(SSM_THREADS) void conv_prepare_kernel(
@@ -30,15 +31,17 @@ __global__ __launch_bounds__(SSM_THREADS) void conv_prepare_kernel(
     const float* __restrict__ tap_bias, const float* __restrict__ dt_bias, const float* __restrict__ neg_a,
     const float* __restrict__ state, long state_ld, int conv_at, const int* __restrict__ row_seq,
     const int* __restrict__ cu_rows, const int* __restrict__ seq_slots, float* __restrict__ u, long ldu, int C, int K,
-    int H, int P) {
-  const long r = blockIdx.x;
+    int H, int P, int row_blocks, int per_thread) {
+  const long r = blockIdx.x / row_blocks;
+  const int block = blockIdx.x % row_blocks;
   const int seq = row_seq[r];
   const int t = (int)(r - cu_rows[seq]);                    // rows of this request that the step brings before this one
   const float* old = state + (long)seq_slots[seq] * state_ld + conv_at;
   const float* row = proj + r * ldp;
   const int inner = H * P;
-  const int c = blockIdx.y * SSM_THREADS + threadIdx.x;
-  if (c < C) {
+  for (int i = 0; i < per_thread; ++i) {
+    const int c = (block * per_thread + i) * SSM_THREADS + threadIdx.x;
+    if (c >= C) break;
     float v[SSM_MAX_TAPS], w[SSM_MAX_TAPS];
 #pragma unroll
     for (int j = 0; j < SSM_MAX_TAPS; ++j) {                // every load first, then the sum in the taps' order
@@ -60,7 +63,7 @@ __global__ __launch_bounds__(SSM_THREADS) void conv_prepare_kernel(
       u[r * ldu + C + c] = y * ssm_softplus(row[dt_off + h] + dt_bias[h]);
     }
   }
-  if (blockIdx.y == 0)
+  if (block == 0)
     for (int h = threadIdx.x; h < H; h += SSM_THREADS)
       u[r * ldu + C + inner + h] = expf(neg_a[h] * ssm_softplus(row[dt_off + h] + dt_bias[h]));
 }
@@ -147,9 +150,12 @@ TIS_EXPORT int tis_conv_prepare(const float* proj, long ldp, int xbc_off, int dt
   if (ldu < (long)C + (long)H * P + H || state_ld < (long)conv_at + (long)(K - 1) * C)
     return tis_fail("conv_prepare: rows of %ld floats for %ld, state lines of %ld for %ld", ldu, (long)C + (long)H * P + H,
                     state_ld, (long)conv_at + (long)(K - 1) * C);
-  conv_prepare_kernel<<<dim3(rows, (C + SSM_THREADS - 1) / SSM_THREADS), SSM_THREADS, 0, stream>>>(
+  const int per_thread = rows >= 512 ? 4 : 1;
+  const int row_blocks = (C + SSM_THREADS * per_thread - 1) / (SSM_THREADS * per_thread);
+  if ((long)rows * row_blocks > 0x7fffffffL) return tis_fail("conv_prepare: %d rows of %d channels in one call", rows, C);
+  conv_prepare_kernel<<<rows * row_blocks, SSM_THREADS, 0, stream>>>(
       proj, ldp, xbc_off, dt_off, taps, tap_bias, dt_bias, neg_a, state, state_ld, conv_at, row_seq, cu_rows, seq_slots, u, ldu,
-      C, K, H, P);
+      C, K, H, P, row_blocks, per_thread);
   return tis_launch_status("conv_prepare");
 }
 

@@ -450,9 +450,9 @@ TIS_EXPORT int tis_head_gate(int dtype, void* x, long ldx, const float* gate, lo
 template <typename T>
 __global__ __launch_bounds__(S32_THREADS) void dyt32_kernel(const float* __restrict__ x, float alpha,
                                                              const float* __restrict__ gain, const float* __restrict__ bias,
-                                                             T* __restrict__ out, long ldo, int D) {
-  const long r = blockIdx.x;
-  const int c = blockIdx.y * S32_THREADS + threadIdx.x;      // grid (rows, blocks of columns): a few rows still fill the chip
+                                                             T* __restrict__ out, long ldo, int D, int row_blocks) {
+  const long r = blockIdx.x / row_blocks;      // grid (rows * blocks of columns, a row's side by side): a few rows still fill the chip
+  const int c = (blockIdx.x % row_blocks) * S32_THREADS + threadIdx.x;
   if (c < D) out[r * ldo + c] = from_f<T>(tanhf(alpha * x[r * D + c]) * gain[c] + (bias ? bias[c] : 0.f));
 }
 
@@ -466,15 +466,15 @@ struct ScaledBranch {
 };
 
 // x <- x + sum over the branches, in place or into out32; `normed` (nullable) gets the dynamic tanh of the new row in
-// the compute type (the norm that the next block, or the model's end, reads the stream through). grid (rows, blocks of
-// columns): every element is on its own, and a step of a few rows still spreads over the chip.
+// the compute type (the norm that the next block, or the model's end, reads the stream through). grid (rows * blocks of
+// columns, a row's blocks side by side): every element is on its own, and a step of a few rows still spreads over the chip.
 template <typename T>
 __global__ __launch_bounds__(S32_THREADS) void scaled_sum_kernel(const float* __restrict__ x, ScaledBranch a, ScaledBranch b,
                                                                   ChosenSum cs, float* __restrict__ out32, int norm_kind,
                                                                   float alpha, const float* __restrict__ gain,
                                                                   const float* __restrict__ nbias, T* __restrict__ normed,
-                                                                  long ldn, int D) {
-  const long r = blockIdx.x;
+                                                                  long ldn, int D, int row_blocks) {
+  const long r = blockIdx.x / row_blocks;
   __shared__ int chosen_id[64];
   __shared__ float chosen_w[64];
   const bool kept = cs.ids && cs.top <= 64;
@@ -485,7 +485,7 @@ __global__ __launch_bounds__(S32_THREADS) void scaled_sum_kernel(const float* __
     }
     __syncthreads();
   }
-  const int c = blockIdx.y * S32_THREADS + threadIdx.x;
+  const int c = (blockIdx.x % row_blocks) * S32_THREADS + threadIdx.x;
   if (c < D) {
     float v = x[r * D + c];
     if (a.y) v += (a.scale ? a.scale[c] : 1.f) * (a.y[r * a.ld + c] + (a.bias ? a.bias[c] : 0.f));
@@ -534,8 +534,10 @@ TIS_EXPORT int tis_dyt32(int dtype, const float* x, float alpha, const float* ga
                          int rows, int D, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || D < 1 || !x || !gain || !out) return tis_fail("dyt32: bad arguments rows=%d width=%d", rows, D);
-  S32_DISPATCH((dyt32_kernel<float><<<dim3(rows, (D + S32_THREADS - 1) / S32_THREADS), S32_THREADS, 0, stream>>>(x, alpha, gain, bias, (float*)out, ldo, D)),
-               (dyt32_kernel<bf16><<<dim3(rows, (D + S32_THREADS - 1) / S32_THREADS), S32_THREADS, 0, stream>>>(x, alpha, gain, bias, (bf16*)out, ldo, D)))
+  const int row_blocks = (D + S32_THREADS - 1) / S32_THREADS;
+  if ((long)rows * row_blocks > 0x7fffffffL) return tis_fail("dyt32: %d rows of %d in one call", rows, D);
+  S32_DISPATCH((dyt32_kernel<float><<<rows * row_blocks, S32_THREADS, 0, stream>>>(x, alpha, gain, bias, (float*)out, ldo, D, row_blocks)),
+               (dyt32_kernel<bf16><<<rows * row_blocks, S32_THREADS, 0, stream>>>(x, alpha, gain, bias, (bf16*)out, ldo, D, row_blocks)))
   return tis_launch_status("dyt32");
 }
 
@@ -552,9 +554,11 @@ TIS_EXPORT int tis_scaled_sum(int dtype, const float* x, const float* y0, long l
     return tis_fail("scaled_sum: norm kind %d (0: none, 3: dynamic tanh, with a gain and an output)", norm_kind);
   const ScaledBranch a{y0, ld0, s0, b0}, b{y1, ld1, s1, b1};
   const ChosenSum cs{ids, weights, top, n_experts, chosen_rows, ldr};
-  const dim3 grid(rows, (D + S32_THREADS - 1) / S32_THREADS);
-  S32_DISPATCH((scaled_sum_kernel<float><<<grid, S32_THREADS, 0, stream>>>(x, a, b, cs, out32, norm_kind, alpha, gain, nbias, (float*)normed, ldn, D)),
-               (scaled_sum_kernel<bf16><<<grid, S32_THREADS, 0, stream>>>(x, a, b, cs, out32, norm_kind, alpha, gain, nbias, (bf16*)normed, ldn, D)))
+  const int row_blocks = (D + S32_THREADS - 1) / S32_THREADS;
+  if ((long)rows * row_blocks > 0x7fffffffL) return tis_fail("scaled_sum: %d rows of %d in one call", rows, D);
+  const int grid = rows * row_blocks;
+  S32_DISPATCH((scaled_sum_kernel<float><<<grid, S32_THREADS, 0, stream>>>(x, a, b, cs, out32, norm_kind, alpha, gain, nbias, (float*)normed, ldn, D, row_blocks)),
+               (scaled_sum_kernel<bf16><<<grid, S32_THREADS, 0, stream>>>(x, a, b, cs, out32, norm_kind, alpha, gain, nbias, (bf16*)normed, ldn, D, row_blocks)))
   return tis_launch_status("scaled_sum");
 }
 
