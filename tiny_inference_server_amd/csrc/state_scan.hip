@@ -44,9 +44,15 @@ __device__ __forceinline__ float sc_log_sigmoid(float z) { return fminf(z, 0.f) 
 // Where a head finds its columns: `qk_group` consecutive heads share one set of query and key columns (1: every head
 // has its own); head h's decay for key channel i lies at h * decay_hs + i * decay_cs of a row's decays (D and 1: one per
 // key channel; 1 and 0: one per head).
+// With one decay per head (decay_cs 0) a row's decays are one number a head: the walk reads that one number from LDS
+// instead of a line of equal ones, keeps one running product instead of one per key channel, and the workspace's
+// `cum` holds [row][H] numbers instead of [row][H*D].
 struct ScanLayout {
   int qk_group, decay_hs, decay_cs;
 };
+__device__ __forceinline__ long cum_at(const ScanLayout& lay, long row, int H, int D, int h, int i) {
+  return lay.decay_cs ? (row * H + h) * D + i : row * H + h;
+}
 
 struct SegArgs {
   int segments;      // most segments of one request in this call; 0: not segmented
@@ -91,8 +97,9 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
   const int col = vb * VB + j;
   const bool col_ok = col < V;
 
+  const bool per_head = KIND == 0 && lay.decay_cs == 0;
   float Sreg[NS], nreg[NS], creg[NS];
-  float m = SEG ? -INFINITY : 0.f, fsum = 0.f;
+  float m = SEG ? -INFINITY : 0.f, fsum = 0.f, cprod = 1.f;
 #pragma unroll
   for (int e = 0; e < NS; ++e) {
     const int i = s * NS + e;
@@ -111,7 +118,8 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
       const bool in = i < D;
       sq[idx] = in ? row[q_off + (h / lay.qk_group) * D + i] * q_scale : 0.f;
       sk[idx] = in ? row[k_off + (h / lay.qk_group) * D + i] : 0.f;
-      if (KIND == 0) sa[idx] = in ? decay[(long)(c0 + c) * ldd + h * lay.decay_hs + i * lay.decay_cs] : 0.f;
+      if (KIND == 0 && (!per_head || i == 0))
+        sa[idx] = in ? decay[(long)(c0 + c) * ldd + h * lay.decay_hs + i * lay.decay_cs] : 0.f;
     }
     for (int idx = t; idx < nc * VB; idx += SC_THREADS) {
       const int c = idx / VB, jj = idx - c * VB;
@@ -139,36 +147,59 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
       const int at = c * DP + s * NS;
       // (channels beyond the head's are zeros in k and q: their state stays zero and adds nothing)
       constexpr int STEP = NS % 4 == 0 ? 4 : 1;      // a thread reads its channels in 16-byte pieces where they allow
+      if (per_head) {
+        const float a = sa[c * DP];                  // the head's one decay of this token
+        cprod *= a;
 #pragma unroll
-      for (int e0 = 0; e0 < NS; e0 += STEP) {
-        float kk[STEP], qq[STEP], aa[STEP];
-        if (STEP == 4) {
-          *reinterpret_cast<float4*>(kk) = *reinterpret_cast<const float4*>(sk + at + e0);
-          *reinterpret_cast<float4*>(qq) = *reinterpret_cast<const float4*>(sq + at + e0);
-          if (KIND == 0) *reinterpret_cast<float4*>(aa) = *reinterpret_cast<const float4*>(sa + at + e0);
-        } else {
-          kk[0] = sk[at + e0];
-          qq[0] = sq[at + e0];
-          if (KIND == 0) aa[0] = sa[at + e0];
-        }
-#pragma unroll
-        for (int u = 0; u < STEP; ++u) {
-          const int e = e0 + u;
-          if (KIND == 0) {
-            Sreg[e] = aa[u] * Sreg[e] + kk[u] * vj;
-            if (SEG) creg[e] *= aa[u];
+        for (int e0 = 0; e0 < NS; e0 += STEP) {
+          float kk[STEP], qq[STEP];
+          if (STEP == 4) {
+            *reinterpret_cast<float4*>(kk) = *reinterpret_cast<const float4*>(sk + at + e0);
+            *reinterpret_cast<float4*>(qq) = *reinterpret_cast<const float4*>(sq + at + e0);
           } else {
-            Sreg[e] = keep * Sreg[e] + take * (kk[u] * vj);
-            nreg[e] = keep * nreg[e] + take * kk[u];
-            nq += nreg[e] * qq[u];
+            kk[0] = sk[at + e0];
+            qq[0] = sq[at + e0];
           }
-          acc += Sreg[e] * qq[u];
-        }
-      }
-      if (KIND == 0 && SEG && vb == 0 && j == 0) {
 #pragma unroll
-        for (int e = 0; e < NS; ++e)
-          if (s * NS + e < D) sg.cum[(long)(c0 + c) * H * D + h * D + s * NS + e] = creg[e];
+          for (int u = 0; u < STEP; ++u) {
+            const int e = e0 + u;
+            Sreg[e] = a * Sreg[e] + kk[u] * vj;
+            acc += Sreg[e] * qq[u];
+          }
+        }
+        if (SEG && vb == 0 && t == 0) sg.cum[cum_at(lay, c0 + c, H, D, h, 0)] = cprod;
+      } else {
+#pragma unroll
+        for (int e0 = 0; e0 < NS; e0 += STEP) {
+          float kk[STEP], qq[STEP], aa[STEP];
+          if (STEP == 4) {
+            *reinterpret_cast<float4*>(kk) = *reinterpret_cast<const float4*>(sk + at + e0);
+            *reinterpret_cast<float4*>(qq) = *reinterpret_cast<const float4*>(sq + at + e0);
+            if (KIND == 0) *reinterpret_cast<float4*>(aa) = *reinterpret_cast<const float4*>(sa + at + e0);
+          } else {
+            kk[0] = sk[at + e0];
+            qq[0] = sq[at + e0];
+            if (KIND == 0) aa[0] = sa[at + e0];
+          }
+#pragma unroll
+          for (int u = 0; u < STEP; ++u) {
+            const int e = e0 + u;
+            if (KIND == 0) {
+              Sreg[e] = aa[u] * Sreg[e] + kk[u] * vj;
+              if (SEG) creg[e] *= aa[u];
+            } else {
+              Sreg[e] = keep * Sreg[e] + take * (kk[u] * vj);
+              nreg[e] = keep * nreg[e] + take * kk[u];
+              nq += nreg[e] * qq[u];
+            }
+            acc += Sreg[e] * qq[u];
+          }
+        }
+        if (KIND == 0 && SEG && vb == 0 && j == 0) {
+#pragma unroll
+          for (int e = 0; e < NS; ++e)
+            if (s * NS + e < D) sg.cum[cum_at(lay, c0 + c, H, D, h, s * NS + e)] = creg[e];
+        }
       }
       part[(c * R + s) * (VB + 1) + j] = acc;
       if (KIND == 1) {
@@ -209,7 +240,7 @@ template <int KIND>
 __global__ __launch_bounds__(SC_THREADS) void segment_states_kernel(float* __restrict__ state, long state_ld,
                                                                     const int* __restrict__ cu_rows,
                                                                     const int* __restrict__ seq_slots, int H, int D,
-                                                                    int V, int n_vb, SegArgs sg) {
+                                                                    int V, int n_vb, SegArgs sg, ScanLayout lay) {
   const int seq = blockIdx.x, h = blockIdx.y;
   const int r0 = cu_rows[seq], r1 = cu_rows[seq + 1];
   if (r0 >= r1) return;
@@ -228,7 +259,7 @@ __global__ __launch_bounds__(SC_THREADS) void segment_states_kernel(float* __res
     const float mine = own[el];
     float next, m_next = 0.f;
     if (KIND == 0) {
-      next = sg.cum[(long)last * H * D + h * D + i] * x + mine;
+      next = sg.cum[cum_at(lay, last, H, D, h, i)] * x + mine;
     } else {
       const float m_own = own[per - 2], f_all = sg.aux[((long)last * H + h) * 3 + 1];
       m_next = fmaxf(f_all + m, m_own);
@@ -278,7 +309,7 @@ __global__ __launch_bounds__(SC_THREADS) void segment_outputs_kernel(const float
     for (int idx = t; idx < nr * D; idx += SC_THREADS) {
       const int r = idx / D, i = idx - r * D;
       float q = proj[(long)(t0 + r) * ldp + q_off + (h / lay.qk_group) * D + i] * q_scale;
-      if (KIND == 0) q *= sg.cum[(long)(t0 + r) * H * D + h * D + i];
+      if (KIND == 0) q *= sg.cum[cum_at(lay, t0 + r, H, D, h, i)];
       qt[r * (D + 1) + i] = q;
     }
     __syncthreads();
@@ -354,7 +385,7 @@ static int launch_scan(bool wide, int ns, dim3 grid, size_t lds, hipStream_t str
   const int n_seqs = grid.x / sg.segments;
   const int elems = D * V + (KIND == 1 ? D : 0);
   segment_states_kernel<KIND><<<dim3(n_seqs, H, (elems + SC_THREADS - 1) / SC_THREADS), SC_THREADS, 0, stream>>>(
-      state, state_ld, cu_rows, seq_slots, H, D, V, n_vb, sg);
+      state, state_ld, cu_rows, seq_slots, H, D, V, n_vb, sg, lay);
   if (tis_launch_status("segment_states")) return -1;
   const size_t lds3 = sizeof(float) * ((size_t)D * SG_COLS + (size_t)SG_ROWS * (D + 1) + SG_ROWS);
   segment_outputs_kernel<KIND><<<dim3(grid.x, H, (V + SG_COLS - 1) / SG_COLS), SC_THREADS, lds3, stream>>>(
