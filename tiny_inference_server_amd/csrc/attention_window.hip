@@ -40,15 +40,14 @@ struct PrepareArgs {
 
 // The norms may also run over all heads of a row at once (whole_norm), and the rotated pairs may be (i, i + rot_dims/2)
 // (pair_half).
-// grid (rows, H + 2 G), one wave each: unit u < H is a query head, u < H + G a key head, else a value head.
-// proj holds the projections of a row in 32-bit: queries at q_off, keys at k_off, values at v_off.
+// One wave's work for unit u of row r: u < H is a query head, u < H + G a key head, else a value head. proj holds the
+// projections of a row in 32-bit: queries at q_off, keys at k_off, values at v_off. whole_q, whole_k: with whole_norm,
+// one over the root mean square of all of the row's queries (keys).
 template <typename T>
-__global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
+__device__ __forceinline__ void prepare_unit(
     const float* __restrict__ proj, long ldp, int q_off, int k_off, int v_off, const int* __restrict__ positions,
-    const int* __restrict__ write_slots, T* __restrict__ plane, T* __restrict__ q_out, long ldq, PrepareArgs a, int H, int G,
-    int KD, int VD, int page_size) {
-  const long r = blockIdx.x;
-  const int u = blockIdx.y, lane = threadIdx.x;
+    const int* __restrict__ write_slots, T* __restrict__ plane, T* __restrict__ q_out, long ldq, const PrepareArgs& a, int H,
+    int G, int KD, int VD, int page_size, long r, int u, int lane, float whole_q, float whole_k) {
   const long page_stride = (long)G * page_size * (KD + VD);
   if (u < H + G) {
     const bool is_q = u < H;
@@ -60,22 +59,7 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
     const float* gain = is_q ? a.q_gain : a.k_gain;
     float inv = 1.f;
     if (gain && a.whole_norm) {
-      // every head's wave sums the whole projection, in the same order: lanes over the channels, then the wave
-      const int n_all = (is_q ? H : G) * KD;
-      const float* all = proj + r * ldp + (is_q ? q_off : k_off);
-      const float* all_bias = is_q ? a.q_bias : a.k_bias;
-      // (four sums side by side, so that a lane's loads are in flight together; the order depends on n_all alone)
-      float part[4] = {0.f, 0.f, 0.f, 0.f};
-      for (int e0 = lane; e0 < n_all; e0 += 4 * TIS_WAVE) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int e = e0 + i * TIS_WAVE;
-          const float v = e < n_all ? all[e] + (all_bias ? all_bias[e] : 0.f) : 0.f;
-          part[i] += v * v;
-        }
-      }
-      const float ss = wave_sum((part[0] + part[1]) + (part[2] + part[3]));
-      inv = 1.f / sqrtf(ss / (float)n_all + a.eps);
+      inv = is_q ? whole_q : whole_k;
       gain += (long)h * KD;
     } else if (gain) {
       float ss = 0.f;
@@ -145,6 +129,47 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
              ws % page_size;
     for (int e = lane; e < VD; e += TIS_WAVE) dst[(long)e * page_size] = from_f<T>((src[e] + (bias ? bias[e] : 0.f)) * inv);
   }
+}
+
+// grid (rows, H + 2 G), one wave each (norms per head or none).
+template <typename T>
+__global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
+    const float* __restrict__ proj, long ldp, int q_off, int k_off, int v_off, const int* __restrict__ positions,
+    const int* __restrict__ write_slots, T* __restrict__ plane, T* __restrict__ q_out, long ldq, PrepareArgs a, int H, int G,
+    int KD, int VD, int page_size) {
+  prepare_unit<T>(proj, ldp, q_off, k_off, v_off, positions, write_slots, plane, q_out, ldq, a, H, G, KD, VD, page_size,
+                  blockIdx.x, blockIdx.y, threadIdx.x, 1.f, 1.f);
+}
+
+// Norms over all heads of a row at once: grid (rows), up to 16 waves a row. The workgroup first sums the squares of
+// the row's queries and of its keys (every element read once; the order of additions depends on the sizes alone), then
+// its waves take the row's units in turn.
+template <typename T>
+__global__ __launch_bounds__(1024) void attention_prepare_row_kernel(
+    const float* __restrict__ proj, long ldp, int q_off, int k_off, int v_off, const int* __restrict__ positions,
+    const int* __restrict__ write_slots, T* __restrict__ plane, T* __restrict__ q_out, long ldq, PrepareArgs a, int H, int G,
+    int KD, int VD, int page_size) {
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  const int t = threadIdx.x, waves = blockDim.x / TIS_WAVE;
+  auto inverse_rms = [&](int off, int n, const float* bias) {
+    const float* all = proj + r * ldp + off;
+    float part[4] = {0.f, 0.f, 0.f, 0.f};        // four sums side by side, so that a thread's loads are in flight together
+    for (int e0 = t; e0 < n; e0 += 4 * blockDim.x) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = e0 + i * blockDim.x;
+        const float v = e < n ? all[e] + (bias ? bias[e] : 0.f) : 0.f;
+        part[i] += v * v;
+      }
+    }
+    return 1.f / sqrtf(block_sum((part[0] + part[1]) + (part[2] + part[3]), red) / (float)n + a.eps);
+  };
+  const float whole_q = a.q_gain ? inverse_rms(q_off, H * KD, a.q_bias) : 1.f;
+  const float whole_k = a.k_gain && write_slots ? inverse_rms(k_off, G * KD, a.k_bias) : 1.f;
+  for (int u = t / TIS_WAVE; u < H + 2 * G; u += waves)
+    prepare_unit<T>(proj, ldp, q_off, k_off, v_off, positions, write_slots, plane, q_out, ldq, a, H, G, KD, VD, page_size, r,
+                    u, t % TIS_WAVE, whole_q, whole_k);
 }
 
 // The same step where all heads share one latent as keys and values. grid (rows, H + 1), one wave each.
@@ -305,6 +330,18 @@ TIS_EXPORT int tis_attention_prepare(int dtype, const float* proj, long ldp, int
   if (write_slots && !plane) return tis_fail("attention_prepare: write slots without pages");
   PrepareArgs a{q_bias, k_bias, v_bias, q_gain, k_gain, q_factor, freqs, rot_dims, eps, value_norm, temp_coef, temp_every,
                 whole_norm, pair_half};
+  if (whole_norm && (q_gain || k_gain)) {
+    const int threads = TIS_WAVE * (H + 2 * G < 16 ? H + 2 * G : 16);
+    if (dtype == TIS_F32)
+      attention_prepare_row_kernel<float><<<rows, threads, 0, stream>>>(proj, ldp, q_off, k_off, v_off, positions, write_slots,
+          (float*)plane, (float*)q_out, ldq, a, H, G, KD, VD, page_size);
+    else if (dtype == TIS_BF16)
+      attention_prepare_row_kernel<bf16><<<rows, threads, 0, stream>>>(proj, ldp, q_off, k_off, v_off, positions, write_slots,
+          (bf16*)plane, (bf16*)q_out, ldq, a, H, G, KD, VD, page_size);
+    else
+      return tis_fail("unknown dtype code %d", dtype);
+    return tis_launch_status("attention_prepare");
+  }
   dim3 grid(rows, H + 2 * G);
   if (dtype == TIS_F32)
     attention_prepare_kernel<float><<<grid, TIS_WAVE, 0, stream>>>(proj, ldp, q_off, k_off, v_off, positions, write_slots,
