@@ -141,7 +141,7 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
                   blockIdx.x, blockIdx.y, threadIdx.x, 1.f, 1.f);
 }
 
-// Norms over all heads of a row at once: grid (rows), up to 16 waves a row. The workgroup first sums the squares of
+// Norms over all heads of a row at once: grid (rows), 4 to 16 waves a row. The workgroup first sums the squares of
 // the row's queries and of its keys (every element read once; the order of additions depends on the sizes alone), then
 // its waves take the row's units in turn.
 template <typename T>
@@ -152,17 +152,20 @@ __global__ __launch_bounds__(1024) void attention_prepare_row_kernel(
   __shared__ float red[16];
   const long r = blockIdx.x;
   const int t = threadIdx.x, waves = blockDim.x / TIS_WAVE;
+  // The first 256 threads sum, whatever the workgroup's size: a row's result is the same bit for bit in a step of few
+  // rows (16 waves a row) and in one of many (4 waves a row).
   auto inverse_rms = [&](int off, int n, const float* bias) {
     const float* all = proj + r * ldp + off;
     float part[4] = {0.f, 0.f, 0.f, 0.f};        // four sums side by side, so that a thread's loads are in flight together
-    for (int e0 = t; e0 < n; e0 += 4 * blockDim.x) {
+    if (t < 256)
+      for (int e0 = t; e0 < n; e0 += 4 * 256) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int e = e0 + i * blockDim.x;
-        const float v = e < n ? all[e] + (bias ? bias[e] : 0.f) : 0.f;
-        part[i] += v * v;
+        for (int i = 0; i < 4; ++i) {
+          const int e = e0 + i * 256;
+          const float v = e < n ? all[e] + (bias ? bias[e] : 0.f) : 0.f;
+          part[i] += v * v;
+        }
       }
-    }
     return 1.f / sqrtf(block_sum((part[0] + part[1]) + (part[2] + part[3]), red) / (float)n + a.eps);
   };
   const float whole_q = a.q_gain ? inverse_rms(q_off, H * KD, a.q_bias) : 1.f;
@@ -331,7 +334,8 @@ TIS_EXPORT int tis_attention_prepare(int dtype, const float* proj, long ldp, int
   PrepareArgs a{q_bias, k_bias, v_bias, q_gain, k_gain, q_factor, freqs, rot_dims, eps, value_norm, temp_coef, temp_every,
                 whole_norm, pair_half};
   if (whole_norm && (q_gain || k_gain)) {
-    const int threads = TIS_WAVE * (H + 2 * G < 16 ? H + 2 * G : 16);
+    const int units = H + 2 * G;
+    const int threads = rows >= 256 ? 256 : TIS_WAVE * (units < 4 ? 4 : units < 16 ? units : 16);
     if (dtype == TIS_F32)
       attention_prepare_row_kernel<float><<<rows, threads, 0, stream>>>(proj, ldp, q_off, k_off, v_off, positions, write_slots,
           (float*)plane, (float*)q_out, ldq, a, H, G, KD, VD, page_size);
