@@ -42,19 +42,12 @@ __global__ __launch_bounds__(SSM_THREADS) void conv_prepare_kernel(
   for (int i = 0; i < per_thread; ++i) {
     const int c = (block * per_thread + i) * SSM_THREADS + threadIdx.x;
     if (c >= C) break;
-    float v[SSM_MAX_TAPS], w[SSM_MAX_TAPS];
-#pragma unroll
-    for (int j = 0; j < SSM_MAX_TAPS; ++j) {                // every load first, then the sum in the taps' order
-      if (j >= K) break;
-      const int back = K - 1 - j;                           // the last tap weighs the row itself
-      v[j] = back <= t ? row[xbc_off + c - (long)back * ldp] : old[(long)(K - 1 + t - back) * C + c];
-      w[j] = taps[(long)c * K + j];
-    }
     float acc = tap_bias ? tap_bias[c] : 0.f;
-#pragma unroll
-    for (int j = 0; j < SSM_MAX_TAPS; ++j) {
-      if (j >= K) break;
-      acc += w[j] * v[j];
+#pragma unroll 4
+    for (int j = 0; j < K; ++j) {
+      const int back = K - 1 - j;                           // the last tap weighs the row itself
+      const float v = back <= t ? row[xbc_off + c - (long)back * ldp] : old[(long)(K - 1 + t - back) * C + c];
+      acc += taps[(long)c * K + j] * v;
     }
     const float y = ssm_silu(acc);
     u[r * ldu + c] = y;
@@ -150,8 +143,12 @@ TIS_EXPORT int tis_conv_prepare(const float* proj, long ldp, int xbc_off, int dt
   if (ldu < (long)C + (long)H * P + H || state_ld < (long)conv_at + (long)(K - 1) * C)
     return tis_fail("conv_prepare: rows of %ld floats for %ld, state lines of %ld for %ld", ldu, (long)C + (long)H * P + H,
                     state_ld, (long)conv_at + (long)(K - 1) * C);
-  const int per_thread = rows >= 512 ? 4 : 1;
-  const int row_blocks = (C + SSM_THREADS * per_thread - 1) / (SSM_THREADS * per_thread);
+  // as many channels a thread as keep the grid at about what the chip holds at once (a workgroup first finds its row's
+  // request and state line, a chain of loads that further rounds of workgroups would pay again)
+  const int blocks_a_row = (C + SSM_THREADS - 1) / SSM_THREADS;
+  int per_thread = (int)(((long)rows * blocks_a_row + 2047) / 2048);
+  per_thread = per_thread < 1 ? 1 : per_thread > blocks_a_row ? blocks_a_row : per_thread;
+  const int row_blocks = (blocks_a_row + per_thread - 1) / per_thread;
   if ((long)rows * row_blocks > 0x7fffffffL) return tis_fail("conv_prepare: %d rows of %d channels in one call", rows, C);
   conv_prepare_kernel<<<rows * row_blocks, SSM_THREADS, 0, stream>>>(
       proj, ldp, xbc_off, dt_off, taps, tap_bias, dt_bias, neg_a, state, state_ld, conv_at, row_seq, cu_rows, seq_slots, u, ldu,
