@@ -81,11 +81,11 @@ def _configs():
     # the state-space mixer alone (no pages at all): one tap (nothing of the convolution to keep), as many groups as heads
     D = config(48, 77, [dense(ssm(2, 12, 16, 1, 4), 32), dense(ssm(4, 6, 4, 4, 1, parts=4), 0), moe(ssm(1, 20, 7, 1, 2), 16, 2, 1)],
                cap=5.0)
-    # attention alone: no mask at all, a chunk longer than any sequence, keys wider and narrower than values, no rotation
-    # entry at all in one layer
+    # attention alone: no mask at all (with keys and values of different sizes and of one size), a chunk longer than any
+    # sequence, keys wider and narrower than values, no rotation entry at all in one layer
     E = config(56, 150, [moe(attention(3, 3, 20, 36, 0.22, dims=None), 24, 7, 3),
                          dense(attention(2, 1, 40, 16, 0.16, chunk=4096, dims=10, base=1e4, factor=8.0), 48),
-                         dense(attention(4, 2, 8, 8, 0.35, chunk=16, dims=2), 0)])
+                         dense(attention(4, 2, 16, 16, 0.3, dims=2), 0)])
     # ones wherever a size may be one: a single head, one key/value head, one group, a state of one number per value
     # channel, values of one channel, one expert, one norm part per channel, chunks longer than a page and a single tap
     F = config(24, 61, [moe(ssm(1, 8, 1, 1, 2), 8, 1, 1), dense(attention(1, 1, 8, 8, 0.4, chunk=19, dims=8, base=100.0), 16),
