@@ -393,7 +393,7 @@ def test_paged_attention_of_drawn_batches(ops_for, monkeypatch, first):
         window = rng.choice([0, 0, 0, rng.randint(5, 900)])
         chunks = random.Random(case + 5000)         # (a draw of its own: the other draws stay what they were)
         if chunks.random() < 0.3:
-            window = -chunks.choice([chunks.randint(1, 900), 32, 64, 200, 1])       # chunks of that many positions
+            window = -chunks.choice([chunks.randint(1, 900), 32, 64, 150, 1])       # chunks of that many positions
         n_heads = n_kv * group
         n_req = rng.randint(1, 4) if rng.random() < 0.8 else rng.randint(10, 24)
         segs = []
