@@ -70,7 +70,7 @@ def chunk_visible(T, size):
 
 def chunked_attention(h, t, pre, m, eps):
     """Grouped-query attention inside chunks of positions: biased projections, an RMS norm over the whole of q and the
-    whole of k (all heads at once), partial rotation in the rotate-half pairing with scaled frequencies."""
+    whole of k (all heads at once), rotation of a head's first channels, paired half the rotated part apart, at frequencies divided by a factor."""
     T = h.shape[0]
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = h @ w64(t, pre + "q").T + w64(t, pre + "q.b")

@@ -1,10 +1,10 @@
 """The Rurorax decoder as a spec of parts.
 
 Token embedding into a 32-bit stream; parallel blocks x <- x + s1 * mixer(h) + s2 * ff(h) in which both sublayers read
-the same h = dyt(x) (dynamic tanh: tanh(alpha x) * gain + bias, no mean and no variance) and s1, s2 are factors per
+the same h = dyt(x) (dynamic tanh: tanh(alpha x) * gain + bias, element by element, without statistics of the row) and s1, s2 are factors per
 channel; a closing dynamic tanh; the embedding table again as the output table; logits capped by cap * tanh(. / cap).
 A layer's mixer is grouped-query attention inside chunks of positions ("attention": biased projections, an RMS norm over
-the whole of a row's queries and of its keys, partial rotation in the rotate-half pairing with scaled frequencies) or a
+the whole of a row's queries and of its keys, rotation of a head's first channels, paired half the rotated part apart, at frequencies divided by a factor) or a
 selective state-space recurrence ("mamba2"). The feed-forward is a gated dense layer with biases and the tanh-form gelu,
 a mixture of gated silu experts with a sigmoid router whose weight scales the expert's input, or absent.
 

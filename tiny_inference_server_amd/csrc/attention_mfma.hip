@@ -45,7 +45,7 @@ static constexpr int DC = (HD + 31) / 32;   // 32-wide chunks of the head for Q.
 static constexpr int DB = HD / 16;          // 16-wide blocks of the head for P.V
 
 // The first key that the row at position p sees. window > 0: the last `window` keys; window < 0: the keys of the row's own
-// chunk of -window positions, chunks counted from position 0; 0: all. Never decreases as p grows, which is what the
+// chunk of -window positions (chunk edges at multiples of that size in the request); 0: all. Never decreases as p grows, which is what the
 // kernels' ranges of steps rest on.
 __device__ __forceinline__ int first_key(int p, int window) {
   if (window > 0) return p - window + 1 > 0 ? p - window + 1 : 0;

@@ -8,7 +8,7 @@
 // of all heads, the values transposed as [value size][slot]. With equal sizes that is the layout the other attention
 // kernels read. The row at position p sees
 // the keys at [max(0, p - window + 1), p] (window 0: all), and with chunk_size c > 0 only those from p - p % c on (the
-// row's own chunk of positions, chunks counted from position 0), found through the request's block table; keys outside are
+// row's own chunk of positions, chunk edges at multiples of the size in the request), found through the request's block table; keys outside are
 // never read, so what a reused page holds cannot reach a result.
 // Norms, angles, scores, the softmax and the weighted sum are 32-bit; `T` is the type of queries and pages.
 #include "common.h"

@@ -304,8 +304,8 @@ def attention_items(seq_rows, group_size: int, tile_cols: int = 0, n_kv_heads: i
 
 def first_key(pos: int, window: int) -> int:
     """The first key that the row at position pos sees, as the matrix-core attention kernels count: window > 0: the
-    last `window` keys; window < 0: the keys of the row's own chunk of -window positions, chunks counted from position
-    0; 0: all."""
+    last `window` keys; window < 0: the keys of the row's own chunk of -window positions, from the last multiple of
+    that size on; 0: all."""
     if window > 0:
         return max(0, pos - window + 1)
     if window < 0:
@@ -978,8 +978,8 @@ class HipOps:
         the general kernel. sink: the softmax's denominator also counts a key of score 0 that has no value. gate
         ([rows, heads] 32-bit, a strided view is fine): head h's result is multiplied by sigmoid(gate[:, h]). Calls with
         a sink or a gate that the matrix-core kernels do not take go to the kernel for keys and values of any sizes.
-        window > 0: a row sees its last `window` keys; window < 0: the keys of its own chunk of -window positions, chunks
-        counted from position 0 (such calls, too, go to the kernel for any sizes where the matrix-core kernels do not
+        window > 0: a row sees its last `window` keys; window < 0: the keys of its own chunk of -window positions, the
+        chunks' edges at multiples of that size in the request (such calls, too, go to the kernel for any sizes where the matrix-core kernels do not
         take them); 0: all.
         """
         group_name = group
@@ -1696,7 +1696,7 @@ class HipOps:
                            scale=None, sink=False, gate=None, chunk=0):
         """Attention of the rows in `batch` over pages whose keys have key_dim and whose values value_dim channels:
         [rows, heads*value_dim]. chunk > 0: a row at position p sees only the keys from p - p % chunk on (its own chunk
-        of positions, counted from position 0). sink: the softmax's denominator also counts a key of score 0 that has no value.
+        of positions; a chunk's edges are multiples of `chunk` in the request). sink: the softmax's denominator also counts a key of score 0 that has no value.
         gate: [rows, heads] 32-bit (a strided view is fine); head h's result is multiplied by sigmoid(gate[:, h])."""
         _rows_view(self._check(q, "q"), "q")
         n = q.shape[0]

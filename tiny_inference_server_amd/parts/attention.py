@@ -348,7 +348,8 @@ class ChunkedAttention:
     at once with a gain of heads * key_dim entries, and so is the whole of its keys, before rotation. The first rot_dims
     channels of every query and key head are rotated in the pairs (i, i + rot_dims / 2) by position * rot_base^(-2i /
     rot_dims) / rot_factor; the other channels pass. score = q.k * scale. The row at position p sees the keys j <= p
-    with floor(j / chunk) = floor(p / chunk), chunks being counted from position 0 of the sequence (chunk 0: all j <= p).
+    with floor(j / chunk) = floor(p / chunk): a chunk's edges are multiples of `chunk` in the request, wherever a prompt
+    was cut into portions (chunk 0: all j <= p).
     out = softmax-weighted values of all heads . Wo^T + bo. Norms, angles, scores and the softmax are 32-bit.
 
     params: width, n_heads, n_kv_heads, key_dim, value_dim, scale, eps, rot_dims, rot_base, rot_factor, chunk. tensors,

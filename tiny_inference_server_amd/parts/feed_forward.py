@@ -138,9 +138,10 @@ class InputWeightedExperts:
     """A mixture of gated experts in which a chosen expert's weight multiplies what the expert reads, not its result.
 
     z = Wr . h (32-bit), s = sigmoid(z) (score "sigmoid") or softmax(z); the `top` experts with the largest s are chosen;
-    a chosen expert's weight is its s, not renormalised; y = sum over the chosen of expert_e(s_e * h) with
-    expert(v) = Wd . (act(Wg . v) * (Wu . v)), no biases. Without biases Wg . (s h) = s (Wg . h), so the weight is
-    applied to the first product's 32-bit results instead of to a rounded copy of the row.
+    a chosen expert's weight is its s as it is (the chosen weights are not scaled to sum to one);
+    y = sum over the chosen of expert_e(s_e * h) with expert(v) = Wd . (act(Wg . v) * (Wu . v)), no biases. Without
+    biases Wg . (s h) = s (Wg . h), so the weight is applied to the first product's 32-bit results instead of to a
+    rounded copy of the row.
 
     params: width, hidden, n_experts, top, score, act. tensors, stored [out, in]: router (n_experts, width),
     gate<e>, up<e> (hidden, width), down<e> (width, hidden).

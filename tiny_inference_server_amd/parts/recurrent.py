@@ -170,18 +170,18 @@ class LightningAttention(_MatrixStateMixer):
 
 @MIXERS.register("selective_state_space")
 class SelectiveStateSpace:
-    """A selective state-space mixer with a scalar decay per head (state-space duality).
+    """A selective state-space mixer with a scalar decay per head.
 
     One input product, laid out [z: inner | x: inner | B: groups*state | C: groups*state | dt: heads] with
-    inner = heads * vdim. x, B and C together pass a causal convolution per channel (`taps` taps with a bias, the last
-    tap on the row itself, zeros before the sequence's start) and silu. dt = softplus(dt + dt_bias). Per head h, which
+    inner = heads * vdim. The columns x, B and C go, channel by channel, through a short convolution over the
+    row and the taps - 1 rows before it (a bias; nothing before a request's first row) and silu. dt = softplus(dt + dt_bias). Per head h, which
     reads the B and C of group h // (heads / groups), with the state S of state x vdim numbers:
     S_t = exp(-exp(a_log[h]) dt_t) S_(t-1) + dt_t B_t x_t^T,  y_t = S_t^T C_t + skip[h] x_t. The heads side by side are
     multiplied by silu(z), then RMS-normed in norm_groups equal parts (each by its own root mean square) with a gain,
     and projected by Wo. Everything between the convolution and the norm is 32-bit.
 
     A request's state line holds S [heads, state, vdim] and after it the convolution's last taps - 1 inputs
-    [taps - 1, channels]; it starts at zero.
+    [taps - 1, channels]; a line that is taken anew is all zeros.
 
     params: width, n_heads, vdim, state, groups, taps, norm_groups, eps. tensors: in (2 inner + 2 groups*state + heads,
     width) and o (width, inner), stored [out, in]; conv (inner + 2 groups*state, taps), conv_bias, dt_bias (heads,),
