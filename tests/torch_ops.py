@@ -318,7 +318,8 @@ class TorchOps:
             n, top = y.ids.shape
             parts = y.results.view(n, top, -1) if y.results is not None else torch.zeros(n, top, x32.shape[1])
             own = (y.ids >= y.n_experts)[:, :, None]
-            y = (y.weights[:, :, None] * torch.where(own, y.rows.float()[:, None, :], parts)).sum(1)
+            extra = y.extra.float() * torch.sigmoid(y.extra_gate.float()) if y.extra is not None else 0.0
+            y = (y.weights[:, :, None] * torch.where(own, y.rows.float()[:, None, :], parts)).sum(1) + extra
         if y is not None:
             y = y.float()[:, :x32.shape[1]]
             if y_rms is not None:
@@ -352,11 +353,21 @@ class TorchOps:
             out[:, out_offset + h * out_group:out_offset + h * out_group + N] = y[:, h].to(out.dtype)
         return out
 
-    def route_topk(self, z, correction, scale, top, score="softmax"):
+    def route_topk(self, z, correction, scale, top, score="softmax", groups=None, renorm=False):
         s = torch.sigmoid(z.float()) if score == "sigmoid" else torch.softmax(z.float(), dim=-1)
         choice = s + correction if correction is not None else s
-        ids = torch.topk(choice, top, dim=-1).indices
-        return ids.to(torch.int32), torch.gather(s, 1, ids) * scale
+        if groups is not None and groups[1] < groups[0]:
+            count, keep = groups
+            n, N = choice.shape
+            best = choice.view(n, count, N // count).max(-1).values
+            kept = torch.zeros(n, count, dtype=torch.bool)
+            kept.scatter_(1, torch.sort(best, dim=-1, descending=True, stable=True).indices[:, :keep], True)
+            choice = torch.where(kept.repeat_interleave(N // count, dim=1), choice, torch.full_like(choice, -math.inf))
+        ids = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+        w = torch.gather(s, 1, ids)
+        if renorm:
+            w = w / (w.sum(-1, keepdim=True) + 1e-20)
+        return ids.to(torch.int32), w * scale
 
     def routed_experts(self, x, ids, weights, w_up, w_down, act="gelu_erf", combine=True):
         from tiny_inference_server_amd.ops.hip_ops import ChosenExperts
@@ -375,19 +386,26 @@ class TorchOps:
         own = (ids >= E)[:, :, None]
         return (weights[:, :, None] * torch.where(own, xf[:, None, :], parts.view(n, top, -1))).sum(1)
 
-    def gated_experts(self, x, ids, weights, w_gate_up, w_down, act="silu"):
+    def gated_experts(self, x, ids, weights, w_gate_up, w_down, act="silu", limit=0.0, weigh="input", n_experts=None):
         from tiny_inference_server_amd.ops.hip_ops import ChosenExperts
-        E, F = w_gate_up.shape[0], w_gate_up.shape[1] // 2
+        E = w_gate_up.shape[0] if w_gate_up is not None else 0
         n, top = ids.shape
         xf = x.float()
         parts = torch.zeros(n * top, x.shape[1])
         for r in range(n):
             for k in range(top):
                 e = int(ids[r, k])
+                if e >= E:
+                    continue            # an identity expert: the sum takes the row itself
                 z = (w_gate_up[e].float() @ xf[r])[None, :]
-                hid = self.gated_act(z, F, act, row_scale=weights[r, k].reshape(1))[0].float()
+                scale = weights[r, k].reshape(1) if weigh == "input" else None
+                hid = self.gated_act(z, w_gate_up.shape[1] // 2, act, row_scale=scale, limit=limit)[0].float()
                 parts[r * top + k] = w_down[e].float() @ hid
-        return ChosenExperts(parts, ids, None, E, x)
+        return ChosenExperts(parts if E else None, ids, None if weigh == "input" else weights, E, x)
+
+    def combine_experts(self, chosen):
+        n, D = chosen.rows.shape
+        return self.residual_norm(torch.zeros(n, D, dtype=torch.float32), chosen)[0]
 
     # ---- blocks whose sublayers read one norm and are summed with a factor per channel ------------------------
     def dyt32(self, x32, alpha, gain, bias=None):
@@ -411,7 +429,7 @@ class TorchOps:
         normed = self.dyt32(x32, norm[1], norm[2], norm[3]) if norm is not None else None
         return x32, normed
 
-    def gated_act(self, z, hidden, act, gate_bias=None, up_bias=None, row_scale=None):
+    def gated_act(self, z, hidden, act, gate_bias=None, up_bias=None, row_scale=None, limit=0.0):
         g, u = z[:, :hidden].float(), z[:, hidden:2 * hidden].float()
         if gate_bias is not None:
             g = g + gate_bias
@@ -419,8 +437,101 @@ class TorchOps:
             u = u + up_bias
         if row_scale is not None:
             g, u = g * row_scale[:, None], u * row_scale[:, None]
+        if act == "clamped_swish":
+            g, u = torch.clamp(g, max=limit), torch.clamp(u, min=-limit, max=limit)
+            return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(self.dtype)
         a = torch.nn.functional.gelu(g, approximate="tanh") if act == "gelu_tanh" else g * torch.sigmoid(g)
         return (a * u).to(self.dtype)
+
+    def activate_rows(self, z, act):
+        zf = z.float()
+        return (torch.relu(zf) ** 2 if act == "relu2" else self._act(zf, act)).to(self.dtype)
+
+    def normed_mean(self, branches, eps):
+        total = 0.0
+        for y, gain in branches:
+            yf = y.float()
+            total = total + yf / torch.sqrt((yf * yf).mean(-1, keepdim=True) + eps) * gain
+        return total / len(branches)
+
+    def lowrank_act(self, low, w2, bias, kind, rate=None, group=1, tau=1.0):
+        z = low.float() @ w2.t()
+        if bias is not None:
+            z = z + bias
+        if kind == "none":
+            return z
+        if kind == "sigmoid_root":
+            return torch.exp(torch.nn.functional.logsigmoid(z) / tau)
+        return torch.exp(-rate.repeat_interleave(group) * torch.nn.functional.softplus(z, threshold=20.0))
+
+    # ---- a gated delta rule -------------------------------------------------------------------------------------
+    def delta_prepare(self, proj, conv_off, beta_off, taps, state, conv_at, batch, n_heads, qk_heads, dim, vdim):
+        n = proj.shape[0]
+        C, K = taps.shape
+        H, G, D, V = n_heads, qk_heads, dim, vdim
+        u = torch.zeros(n, C + H, dtype=torch.float32)
+        cu, slots = batch.cu_rows.tolist(), batch.seq_slots.tolist()
+        for k in range(batch.n_seqs):
+            first, rows = cu[k], cu[k + 1] - cu[k]
+            if rows == 0:
+                continue
+            old = state[slots[k], conv_at:conv_at + (K - 1) * C].view(K - 1, C)
+            seq = torch.cat((old, proj[first:first + rows, conv_off:conv_off + C].float()), dim=0)
+            acc = torch.zeros(rows, C)
+            for j in range(K):
+                acc = acc + seq[j:j + rows] * taps[:, j]
+            y = acc * torch.sigmoid(acc)
+            qk = y[:, :2 * G * D].view(rows, 2 * G, D)
+            qk = qk / torch.sqrt((qk * qk).sum(-1, keepdim=True) + 1e-6)
+            qk[:, :G] *= D ** -0.5
+            u[first:first + rows, :2 * G * D] = qk.reshape(rows, -1)
+            u[first:first + rows, 2 * G * D:C] = y[:, 2 * G * D:]
+            u[first:first + rows, C:] = torch.sigmoid(proj[first:first + rows, beta_off:beta_off + H].float())
+        return u
+
+    def delta_scan(self, u, q_off, k_off, v_off, beta_off, decay, state, batch, n_heads, qk_heads, dim, vdim):
+        H, G, D, V = n_heads, qk_heads, dim, vdim
+        n = u.shape[0]
+        out = torch.zeros(n, H * V, dtype=torch.float32)
+        cu, slots = batch.cu_rows.tolist(), batch.seq_slots.tolist()
+        rep = H // G
+        for s in range(batch.n_seqs):
+            S = state[slots[s], :H * D * V].view(H, D, V)
+            for r in range(cu[s], cu[s + 1]):
+                q = u[r, q_off:q_off + G * D].view(G, D).repeat_interleave(rep, dim=0)
+                k = u[r, k_off:k_off + G * D].view(G, D).repeat_interleave(rep, dim=0)
+                v = u[r, v_off:v_off + H * V].view(H, V)
+                beta = u[r, beta_off:beta_off + H]
+                S.mul_(decay[r].view(H, D, 1))
+                w = beta[:, None] * (v - torch.einsum("hdv,hd->hv", S, k))
+                S.add_(k[:, :, None] * w[:, None, :])
+                out[r] = torch.einsum("hdv,hd->hv", S, q).reshape(-1)
+        return out
+
+    # ---- attention whose weights are sigmoids mixed across the heads --------------------------------------------
+    def mixed_sigmoid_attention(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, chunk,
+                                scale, softcap, head_bias, talk):
+        n = q.shape[0]
+        H, G, kd, vd = n_heads, n_kv_heads, key_dim, value_dim
+        tables = batch.block_tables[group]
+        pages = plane.view(plane.shape[0], -1)
+        keys = pages[:, :G * page_size * kd].view(-1, G, page_size, kd)
+        vals = pages[:, G * page_size * kd:].view(-1, G, vd, page_size)
+        out = torch.zeros(n, H * vd, dtype=torch.float32, device=q.device)
+        pos, seq = batch.positions.tolist(), batch.row_seq.tolist()
+        for r in range(n):
+            p = pos[r]
+            first = p - p % chunk if chunk > 0 else 0
+            js = torch.arange(first, p + 1)
+            pg = tables[seq[r]].long()[js // page_size]
+            k = keys[pg, :, js % page_size].float().repeat_interleave(H // G, dim=1)      # [keys, H, kd]
+            v = vals[pg, :, :, js % page_size].float().repeat_interleave(H // G, dim=1)   # [keys, H, vd]
+            sc = torch.einsum("jhd,hd->hj", k, q[r].float().view(H, kd)) * scale
+            if softcap:
+                sc = softcap * torch.tanh(sc / softcap)
+            w = talk.float() @ torch.sigmoid(sc + head_bias[:, None])
+            out[r] = torch.einsum("hj,jhv->hv", w, v).reshape(-1)
+        return out.to(q.dtype)
 
     def softcap(self, z, cap):
         z.copy_(cap * torch.tanh(z / cap))

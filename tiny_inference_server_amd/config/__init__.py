@@ -4,3 +4,4 @@ from .registry import Registry
 from .fikevik_config import FikevikConfig
 from .fipuzen_config import FipuzenConfig
 from .rurorax_config import RuroraxConfig
+from .fesupel_config import FesupelConfig

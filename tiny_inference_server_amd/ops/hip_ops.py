@@ -450,6 +450,8 @@ class ChosenExperts(NamedTuple):
     weights: torch.Tensor               # [rows, top] 32-bit
     n_experts: int                      # ids from here on are identity experts
     rows: torch.Tensor                  # [rows, width] in the compute type: what the feed-forward read
+    extra: Optional[torch.Tensor] = None        # [rows, width] 32-bit: what every row adds beside its choices (a shared
+    extra_gate: Optional[torch.Tensor] = None   # expert), times sigmoid(extra_gate [rows, 1] 32-bit, a strided view is fine)
 
 
 class AttentionLaunch(NamedTuple):

@@ -174,10 +174,29 @@ class WindowedQkNormAttention:
         return self.ops.linear(self.core(proj, ctx), self.w_o, residual=residual)
 
 
-def _rotary_frequencies(ops, dims: int, base: float):
-    """base^(-2i/dims) for the pairs i < dims/2, on the device in 32-bit (computed in 64-bit)."""
+def banded_frequencies(dims: int, base: float, bands=None):
+    """base^(-2i/dims) for the pairs i < dims/2 in 64-bit. bands = (factor, low, high, original) slows the long waves:
+    with wavelength l = 2 pi / f, a pair with l < original / high keeps f, one with l > original / low turns at
+    f / factor, and between the two f is blended with f / factor by s = (original / l - low) / (high - low):
+    (1 - s) f / factor + s f."""
+    import math
     i = torch.arange(dims // 2, dtype=torch.float64)
-    return (float(base) ** (-2.0 * i / max(1, dims))).to(torch.float32).to(ops.device)
+    f = float(base) ** (-2.0 * i / max(1, dims))
+    if bands is None:
+        return f
+    factor, low, high, original = (float(b) for b in bands)
+    wave = 2.0 * math.pi / f
+    if high == low:
+        s = (wave < original / high).to(torch.float64)
+    else:
+        s = torch.clamp((original / wave - low) / (high - low), 0.0, 1.0)
+    blended = (1.0 - s) * f / factor + s * f
+    return torch.where(wave < original / high, f, torch.where(wave > original / low, f / factor, blended))
+
+
+def _rotary_frequencies(ops, dims: int, base: float, bands=None):
+    """The rotation's frequencies on the device in 32-bit (computed in 64-bit)."""
+    return banded_frequencies(dims, base, bands).to(torch.float32).to(ops.device)
 
 
 @MIXERS.register("sink_gated_attention")
@@ -429,6 +448,84 @@ class ChunkedAttention:
     def forward32(self, x, ctx):
         y, bias = self.forward_parts(x, ctx)
         return y + bias
+
+    def forward(self, x, ctx, residual=None):
+        y = self.forward32(x, ctx)
+        if residual is not None:
+            y = y + residual.to(torch.float32)
+        return y.to(self.ops.dtype)
+
+
+@MIXERS.register("sigmoid_mixed_attention")
+class SigmoidMixedAttention:
+    """Grouped-query attention inside chunks of positions whose weights are sigmoids, not a softmax, and are mixed across
+    the heads before they meet the values.
+
+    q = x.Wq^T + bq, k = x.Wk^T + bk, v = x.Wv^T + bv. The first rot_dims channels of every query and key head are
+    rotated in the pairs (i, i + rot_dims / 2) by position * f_i (f from `banded_frequencies`); the other channels pass.
+    s = q.k * scale, then s <- softcap * tanh(s / softcap) (softcap 0: as it is). The row at position p sees the keys
+    j <= p with floor(j / chunk) = floor(p / chunk) (chunk 0: all j <= p); a seen key's weight for head g is
+    w_g = sigmoid(s + head_bias[g]), each key on its own. Head h then uses sum_g talk[h, g] * w_g on the values of its
+    own key/value head; out = heads . Wo^T. Angles, scores and weights are 32-bit.
+
+    params: width, n_heads, n_kv_heads, key_dim, value_dim, scale, softcap, chunk, rot_dims, rot_base, rot_bands
+    ((factor, low, high, original) or None). tensors, stored [out, in]: q (heads*key_dim, width), k (kv_heads*key_dim,
+    width), v (kv_heads*value_dim, width), q_bias, k_bias, v_bias, head_bias (heads,), talk (heads, heads),
+    o (width, heads*value_dim).
+    """
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, H, G, kd, vd = (params[k] for k in ("width", "n_heads", "n_kv_heads", "key_dim", "value_dim"))
+        return {"q": (H * kd, w), "k": (G * kd, w), "v": (G * vd, w), "q_bias": (H * kd,), "k_bias": (G * kd,),
+                "v_bias": (G * vd,), "head_bias": (H,), "talk": (H, H), "o": (w, H * vd)}
+
+    @classmethod
+    def cache_need(cls, params):
+        # every key is kept: a chunk's keys are found through the same block table as any others
+        return PagedKvNeed(params["n_kv_heads"], params["key_dim"], 0, value_dim=params["value_dim"])
+
+    def __init__(self, spec, tensors, ops):
+        from .base import to_gain
+        p = spec.params
+        self.ops = ops
+        self.H, self.G, self.kd, self.vd = int(p["n_heads"]), int(p["n_kv_heads"]), int(p["key_dim"]), int(p["value_dim"])
+        if self.H % self.G:
+            raise ValueError(f"{self.H} query heads are not a multiple of {self.G} key/value heads")
+        self.scale, self.softcap, self.chunk = float(p["scale"]), float(p.get("softcap", 0.0)), int(p.get("chunk", 0))
+        self.rot_dims = int(p.get("rot_dims", 0))
+        if self.rot_dims % 2 or self.rot_dims > self.kd or self.chunk < 0 or self.softcap < 0:
+            raise ValueError(f"{self.rot_dims} rotated channels of a head of {self.kd} (an even number, at most the head), "
+                             f"chunks of {self.chunk}, a cap of {self.softcap}")
+        self.freqs = _rotary_frequencies(ops, self.rot_dims, float(p.get("rot_base", 10000.0)), p.get("rot_bands"))
+        mats = [tensors.of(spec, k) for k in ("q", "k", "v")]
+        self.input_rows = torch.cat(mats, dim=0)        # as stored: a block may fuse them into a wider product
+        self.k_at = mats[0].shape[0]
+        self.v_at = self.k_at + mats[1].shape[0]
+        self._w_in = None
+        self.q_bias, self.k_bias, self.v_bias = (to_gain(ops, tensors.of(spec, k)) for k in ("q_bias", "k_bias", "v_bias"))
+        self.head_bias = to_gain(ops, tensors.of(spec, "head_bias"))
+        self.talk = to_gain(ops, tensors.of(spec, "talk"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+
+    def core(self, proj, ctx):
+        ops, b = self.ops, ctx.batch
+        q = ops.attention_prepare(proj, 0, self.k_at, self.v_at, b.positions, b.write_slots[ctx.group], ctx.plane, self.H,
+                                  self.G, self.kd, self.vd, ctx.page_size, freqs=self.freqs, rot_dims=self.rot_dims,
+                                  write_cache=ctx.writes_cache, value_norm=False, q_bias=self.q_bias, k_bias=self.k_bias,
+                                  v_bias=self.v_bias, pair_half=True)
+        return ops.mixed_sigmoid_attention(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, self.vd, ctx.page_size,
+                                           self.chunk, self.scale, self.softcap, self.head_bias, self.talk)
+
+    def forward_projected(self, proj, ctx):
+        """From this mixer's columns of a 32-bit input product to its result in 32-bit."""
+        return self.ops.linear(self.core(proj, ctx), self.w_o, out_dtype=torch.float32)
+
+    def forward32(self, x, ctx):
+        if self._w_in is None:
+            self._w_in = to_compute(self.ops, self.input_rows)
+        return self.forward_projected(self.ops.linear(x, self._w_in, out_dtype=torch.float32), ctx)
 
     def forward(self, x, ctx, residual=None):
         y = self.forward32(x, ctx)

@@ -187,3 +187,112 @@ class InputWeightedExperts:
         if residual is not None:
             y = y + residual.to(torch.float32)
         return y.to(self.ops.dtype)
+
+
+@FEED_FORWARDS.register("activated_dense")
+class ActivatedDense:
+    """y = Wd . act(Wu . h), no gate and no biases. params: width, hidden, act ("relu2": the square of relu, or
+    "gelu_tanh", "silu"). tensors, stored [out, in]: up (hidden, width), down (width, hidden)."""
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        d, f = params["width"], params["hidden"]
+        return {"up": (f, d), "down": (d, f)}
+
+    def __init__(self, spec, tensors, ops):
+        self.ops = ops
+        self.act = str(spec.params.get("act", "relu2"))
+        self.w_up = to_compute(ops, tensors.of(spec, "up"))
+        self.w_down = to_compute(ops, tensors.of(spec, "down"))
+
+    def forward32(self, rows):
+        ops = self.ops
+        hidden = ops.activate_rows(ops.linear(rows, self.w_up, out_dtype=torch.float32), self.act)
+        return ops.linear(hidden, self.w_down, out_dtype=torch.float32)
+
+    def forward(self, x, residual=None):
+        y = self.forward32(x)
+        if residual is not None:
+            y = y + residual.to(torch.float32)
+        return y.to(self.ops.dtype)
+
+
+@FEED_FORWARDS.register("grouped_choice_experts")
+class GroupedChoiceExperts:
+    """A mixture of clamped gated experts whose router first narrows the choice to a few groups of neighbours, with
+    identity experts and an optional shared expert behind a gate.
+
+    z = Wr . h (32-bit), s = softmax(z) over all router outputs. The choice looks at s + correction: the outputs form
+    `groups` equal runs of neighbours, a group's score is its largest s + correction, only outputs of the `keep` best
+    groups can be chosen, and of those the `top` largest s + correction are. A chosen output's weight is its s (without
+    the correction) divided by the sum of the chosen s (+ 1e-20). Output e < n_experts is the expert
+    Wd[e] . (g sigmoid(1.702 g) (u + 1)) with g = min(Wg[e] . h, limit), u = clamp(Wu[e] . h, -limit, limit), no biases;
+    the last n_identity outputs are identity experts without tensors whose result is h itself. A shared expert of the
+    same form (sizes and limit of its own) runs for every row and is added times sigmoid(wsg . h), one number a row.
+    y = the weighted sum of the chosen + the gated shared expert, in 32-bit.
+
+    params: width, hidden, limit, n_experts, n_identity, top, groups, keep, shared_hidden (0: none), shared_limit.
+    tensors, stored [out, in]: router (n_experts + n_identity, width), correction (n_experts + n_identity,), gate<e>,
+    up<e> (hidden, width), down<e> (width, hidden), and with a shared expert shared_gate, shared_up (shared_hidden,
+    width), shared_down (width, shared_hidden), shared_sg (1, width).
+    """
+    graph_safe = True
+    sums_in_residual = True     # forward32(x, combine=False) is there
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, f, E, I = params["width"], params["hidden"], params["n_experts"], params.get("n_identity", 0)
+        shapes = {"router": (E + I, w), "correction": (E + I,)}
+        for e in range(E):
+            shapes.update({f"gate{e}": (f, w), f"up{e}": (f, w), f"down{e}": (w, f)})
+        fs = params.get("shared_hidden", 0)
+        if fs:
+            shapes.update({"shared_gate": (fs, w), "shared_up": (fs, w), "shared_down": (w, fs), "shared_sg": (1, w)})
+        return shapes
+
+    def __init__(self, spec, tensors, ops):
+        from .base import to_gain
+        p = spec.params
+        self.ops = ops
+        self.E, self.I, self.top = int(p["n_experts"]), int(p.get("n_identity", 0)), int(p["top"])
+        self.groups, self.keep = int(p.get("groups", 1)), int(p.get("keep", 1))
+        n = self.E + self.I
+        if not 1 <= self.top <= n or self.groups < 1 or n % self.groups or not 1 <= self.keep <= self.groups \
+                or self.top > self.keep * (n // self.groups):
+            raise ValueError(f"{self.top} of {self.E} + {self.I} experts in {self.groups} groups of which {self.keep} are kept")
+        self.limit, self.F = float(p.get("limit", 0.0)), int(p.get("hidden", 0))
+        self.w_router = to_compute(ops, tensors.of(spec, "router"))
+        self.correction = to_gain(ops, tensors.of(spec, "correction"))
+        self.w_gate_up = self.w_down = None
+        if self.E:
+            self.w_gate_up = to_compute(ops, torch.stack([torch.cat((tensors.of(spec, f"gate{e}"), tensors.of(spec, f"up{e}")), dim=0)
+                                                          for e in range(self.E)]))
+            self.w_down = to_compute(ops, torch.stack([tensors.of(spec, f"down{e}") for e in range(self.E)]))
+        self.Fs = int(p.get("shared_hidden", 0))
+        if self.Fs:
+            self.shared_limit = float(p["shared_limit"])
+            # one product for the shared expert's gate, its other factor, and the number that gates its result
+            self.w_shared_in = to_compute(ops, torch.cat([tensors.of(spec, k) for k in ("shared_gate", "shared_up", "shared_sg")], dim=0))
+            self.w_shared_down = to_compute(ops, tensors.of(spec, "shared_down"))
+
+    def forward32(self, x, combine=True):
+        """combine=False: the experts' results before the sum over a row's choices (and the shared expert's before its
+        gate), as a `ChosenExperts` for a residual sum that takes the sum itself."""
+        ops = self.ops
+        z = ops.linear(x, self.w_router, out_dtype=torch.float32)
+        ids, weights = ops.route_topk(z, self.correction, 1.0, self.top, groups=(self.groups, self.keep), renorm=True)
+        chosen = ops.gated_experts(x, ids, weights, self.w_gate_up, self.w_down, "clamped_swish", limit=self.limit,
+                                   weigh="output", n_experts=self.E)
+        if self.Fs:
+            zs = ops.linear(x, self.w_shared_in, out_dtype=torch.float32)
+            hidden = ops.gated_act(zs, self.Fs, "clamped_swish", limit=self.shared_limit)
+            shared = ops.linear(hidden, self.w_shared_down, out_dtype=torch.float32)
+            chosen = chosen._replace(extra=shared, extra_gate=zs[:, 2 * self.Fs:2 * self.Fs + 1])
+        return chosen if not combine else ops.combine_experts(chosen)
+
+    def forward(self, x, residual=None):
+        y = self.forward32(x)
+        if residual is not None:
+            y = y + residual.to(torch.float32)
+        return y.to(self.ops.dtype)

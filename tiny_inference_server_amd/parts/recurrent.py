@@ -241,3 +241,97 @@ class SelectiveStateSpace:
     def forward(self, x, ctx, residual=None):
         proj = self.ops.linear(x, self.w_in, out_dtype=torch.float32)
         return self.ops.linear(self.core(proj, ctx), self.w_o, residual=residual)
+
+
+@MIXERS.register("gated_delta_rule")
+class GatedDeltaRule:
+    """A matrix state per head that is corrected towards each new value instead of only added to, with a decay per key
+    channel.
+
+    q = x.Wq^T and k = x.Wk^T (qk_heads x dim), v = x.Wv^T (heads x vdim), no biases; head h reads the q and k of
+    qk head h // (heads / qk_heads). q, k and v go, channel by channel, through a short convolution over the row and
+    the taps - 1 rows before it (no bias; nothing before a request's first row) and silu. q and k are then made unit
+    vectors per head, x / sqrt(sum x^2 + 1e-6), and q is multiplied by dim^(-1/2). beta = sigmoid(x.Wb^T), one per head.
+    a = exp(-exp(a_log[h]) * softplus((x.Wa1^T).Wa2^T + dt_bias)), one per head and key channel. Per head and row:
+    S <- diag(a) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q (the row reads what it has just written).
+    Each head's o is divided by its root mean square over vdim (eps under the root), times a gain of vdim entries that
+    the heads share, times sigmoid((x.Wg1^T).Wg2^T); then Wo. Everything between the convolution and the gate is 32-bit.
+
+    A request's state line holds S [heads, dim, vdim] and after it the convolution's last taps - 1 inputs
+    [taps - 1, channels]; a line that is taken anew is all zeros.
+
+    params: width, n_heads, qk_heads, dim, vdim, taps, decay_rank, gate_rank, eps. tensors, stored [out, in]: q, k
+    (qk_heads*dim, width), v (heads*vdim, width), q_conv, k_conv, v_conv ([channels, taps], the last column weighs the
+    row itself), b (heads, width), a_log (heads,), a1 (decay_rank, width), a2 (heads*dim, decay_rank), dt_bias
+    (heads*dim,), g1 (gate_rank, width), g2 (heads*vdim, gate_rank), norm (vdim,), o (width, heads*vdim).
+    """
+    graph_safe = True
+
+    @classmethod
+    def _sizes(cls, params):
+        H, G, D, V, K = (int(params[k]) for k in ("n_heads", "qk_heads", "dim", "vdim", "taps"))
+        return H, G, D, V, K, 2 * G * D + H * V
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        H, G, D, V, K, C = cls._sizes(params)
+        w, ra, rg = params["width"], params["decay_rank"], params["gate_rank"]
+        return {"q": (G * D, w), "k": (G * D, w), "v": (H * V, w), "q_conv": (G * D, K), "k_conv": (G * D, K),
+                "v_conv": (H * V, K), "b": (H, w), "a_log": (H,), "a1": (ra, w), "a2": (H * D, ra), "dt_bias": (H * D,),
+                "g1": (rg, w), "g2": (H * V, rg), "norm": (V,), "o": (w, H * V)}
+
+    @classmethod
+    def cache_need(cls, params):
+        H, G, D, V, K, C = cls._sizes(params)
+        return StateNeed((H * D * V + (K - 1) * C,), "float32")
+
+    def __init__(self, spec, tensors, ops):
+        p = spec.params
+        self.ops = ops
+        self.H, self.G, self.D, self.V, self.K, self.C = self._sizes(p)
+        if self.H % self.G:
+            raise ValueError(f"{self.H} heads are not a multiple of {self.G} query/key heads")
+        self.eps = float(p["eps"])
+        self.ra, self.rg = int(p["decay_rank"]), int(p["gate_rank"])
+        keys = ("q", "k", "v", "b", "a1", "g1")
+        mats = [tensors.of(spec, k) for k in keys]
+        self.input_rows = torch.cat(mats, dim=0)        # as stored: a block may fuse them into a wider product
+        self.at, at = {}, 0
+        for k, m in zip(keys, mats):
+            self.at[k] = at
+            at += m.shape[0]
+        self._w_in = None
+        self.taps = to_gain(ops, torch.cat([tensors.of(spec, k) for k in ("q_conv", "k_conv", "v_conv")], dim=0))
+        self.rate = torch.exp(to_gain(ops, tensors.of(spec, "a_log")))          # the decay's rate per head, 32-bit
+        self.w_a2, self.dt_bias = to_gain(ops, tensors.of(spec, "a2")), to_gain(ops, tensors.of(spec, "dt_bias"))
+        self.w_g2 = to_gain(ops, tensors.of(spec, "g2"))
+        self.norm_gain = to_gain(ops, tensors.of(spec, "norm"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+        self.conv_at = self.H * self.D * self.V                                  # where the line's convolution inputs start
+
+    def core(self, proj, ctx):
+        ops, b, at = self.ops, ctx.batch, self.at
+        H, G, D, V, C = self.H, self.G, self.D, self.V, self.C
+        # u: the convolved q (unit, scaled), k (unit), v side by side, then beta
+        u = ops.delta_prepare(proj, at["q"], at["b"], self.taps, ctx.state, self.conv_at, b, H, G, D, V)
+        ops.conv_state_update(proj, at["q"], C, self.K, ctx.state, self.conv_at, b)      # after the rows have read the line
+        decay = ops.lowrank_act(proj[:, at["a1"]:at["a1"] + self.ra], self.w_a2, self.dt_bias, "exp_softplus",
+                                rate=self.rate, group=D)
+        o = ops.delta_scan(u, 0, G * D, 2 * G * D, C, decay, ctx.state, b, H, G, D, V)
+        gate = ops.lowrank_act(proj[:, at["g1"]:at["g1"] + self.rg], self.w_g2, None, "none")
+        return ops.head_norm_gate(o, gate, self.norm_gain, H, V, self.eps, "sigmoid")
+
+    def forward_projected(self, proj, ctx):
+        """From this mixer's columns of a 32-bit input product to its result in 32-bit."""
+        return self.ops.linear(self.core(proj, ctx), self.w_o, out_dtype=torch.float32)
+
+    def forward32(self, x, ctx):
+        if self._w_in is None:
+            self._w_in = to_compute(self.ops, self.input_rows)
+        return self.forward_projected(self.ops.linear(x, self._w_in, out_dtype=torch.float32), ctx)
+
+    def forward(self, x, ctx, residual=None):
+        y = self.forward32(x, ctx)
+        if residual is not None:
+            y = y + residual.to(torch.float32)
+        return y.to(self.ops.dtype)

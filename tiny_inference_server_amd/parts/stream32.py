@@ -58,7 +58,13 @@ class RmsNorm:
         self.eps = float(spec.params["eps"])
         self.gain = to_gain(ops, tensors.of(spec, "gain"))
 
+    def fused(self):
+        """(kind, gain, bias, eps) for a residual sum that applies this norm to its result."""
+        return "rms", self.gain, None, self.eps
+
     def __call__(self, x):
+        if isinstance(x, Stream32) and x.normed_by is self:
+            return x.rows               # the block before has applied this norm in its last kernel
         return self.ops.rmsnorm32(x.full if isinstance(x, Stream32) else x, self.gain, self.eps)
 
 
