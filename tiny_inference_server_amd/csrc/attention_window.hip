@@ -400,3 +400,142 @@ TIS_EXPORT int tis_attention_window(int dtype, const void* q, long ldq, const vo
     return tis_fail("unknown dtype code %d", dtype);
   return tis_launch_status("attention_window");
 }
+
+// ---- attention whose weights are sigmoids mixed across the heads ----------------------------------------------------
+//
+// For the row at position p and every key j it sees (j <= p, and with chunk_size c > 0 only j >= p - p % c):
+//   s_g = q_g . k_kv(g) * scale;  s_g <- cap * tanh(s_g / cap) (cap 0: as it is);  w_g = sigmoid(s_g + head_bias[g]);
+//   m_h = sum_g talk[h][g] * w_g;  out_h = sum_j m_h(j) * v_kv(h)(j).
+// Nothing is normalised over the keys, so a row's result is a plain sum over its keys and may be cut anywhere: with
+// n_splits > 1 workgroup (row, s) takes the key blocks s, s + n_splits, ... and leaves its part in `partial`
+// [rows][n_splits][H * VD] (32-bit), which attention_mixed_merge_kernel adds up in the order of the splits.
+//
+// One workgroup per (row, split). A block of `block` keys at a time: every (head, key) score by one thread into LDS, the
+// mixture of the heads' weights into LDS, then a thread per (head, value channel) adds the block's weighted values.
+// LDS (floats): q of all heads [H * KD] | talk [H * H] | weights [H * block] | mixed [H * block].
+static constexpr int AM_PER = 16;      // (head, value channel) outputs a thread may own: H * VD <= 16 * 256
+
+template <typename T>
+__global__ __launch_bounds__(AW_THREADS) void attention_mixed_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ plane, const int* __restrict__ block_tables, int bt_ld,
+    const int* __restrict__ row_seq, const int* __restrict__ positions, T* __restrict__ out, long ldo,
+    float* __restrict__ partial, int n_splits, int H, int G, int KD, int VD, int page_size, int chunk_size, float scale,
+    float softcap, const float* __restrict__ head_bias, const float* __restrict__ talk, int block) {
+  extern __shared__ float am_lds[];
+  float* qs = am_lds;
+  float* tk = qs + H * KD;
+  float* wr = tk + H * H;
+  float* wm = wr + H * block;
+  const long r = blockIdx.x;
+  const int split = blockIdx.y, t = threadIdx.x;
+  const int group_size = H / G;
+  const int pos = positions[r];
+  const int* bt = block_tables + (long)row_seq[r] * bt_ld;
+  const int first = chunk_size > 0 ? pos - pos % chunk_size : 0;
+  const int end = pos + 1;
+  for (int d = t; d < H * KD; d += AW_THREADS) qs[d] = to_f(q[r * ldq + d]) * scale;
+  for (int d = t; d < H * H; d += AW_THREADS) tk[d] = talk[d];
+  __syncthreads();
+  const long page_stride = (long)G * page_size * (KD + VD);
+  const long v_base = (long)G * page_size * KD;
+  const int n_out = H * VD;
+  float acc[AM_PER];
+#pragma unroll
+  for (int u = 0; u < AM_PER; ++u) acc[u] = 0.f;
+  const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+  for (int c0 = first + split * block; c0 < end; c0 += n_splits * block) {
+    const int n = min(block, end - c0);
+    for (int i = t; i < H * n; i += AW_THREADS) {
+      const int g = i / n, k = i % n, j = c0 + k;
+      const T* kp = plane + (long)bt[j / page_size] * page_stride + (long)(g / group_size) * page_size * KD +
+                    (long)(j % page_size) * KD;
+      const float* qg = qs + g * KD;
+      float s = 0.f;
+      for (int e = 0; e < KD; ++e) s += qg[e] * to_f(kp[e]);
+      if (softcap > 0.f) s = softcap * tanhf(s * inv_cap);
+      wr[g * block + k] = 1.f / (1.f + expf(-(s + head_bias[g])));
+    }
+    __syncthreads();
+    for (int i = t; i < H * n; i += AW_THREADS) {
+      const int h = i / n, k = i % n;
+      float m = 0.f;
+      for (int g = 0; g < H; ++g) m += tk[h * H + g] * wr[g * block + k];
+      wm[h * block + k] = m;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < AM_PER; ++u) {
+      const int o = t + u * AW_THREADS;
+      if (o < n_out) {
+        const int h = o / VD, c = o % VD;
+        const long v_off = v_base + ((long)(h / group_size) * VD + c) * page_size;
+        const float* w = wm + h * block;
+        float a = acc[u];
+        for (int k = 0; k < n; ++k) {
+          const int j = c0 + k;
+          a += w[k] * to_f(plane[(long)bt[j / page_size] * page_stride + v_off + (j % page_size)]);
+        }
+        acc[u] = a;
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int u = 0; u < AM_PER; ++u) {
+    const int o = t + u * AW_THREADS;
+    if (o < n_out) {
+      if (n_splits > 1) partial[(r * n_splits + split) * n_out + o] = acc[u];
+      else out[r * ldo + o] = from_f<T>(acc[u]);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(AW_THREADS) void attention_mixed_merge_kernel(const float* __restrict__ partial, int n_splits,
+                                                                           T* __restrict__ out, long ldo, int rows,
+                                                                           int n_out) {
+  const long i = (long)blockIdx.x * AW_THREADS + threadIdx.x;
+  if (i >= (long)rows * n_out) return;
+  const long r = i / n_out;
+  const int o = (int)(i % n_out);
+  float a = 0.f;
+  for (int s = 0; s < n_splits; ++s) a += partial[(r * n_splits + s) * n_out + o];
+  out[r * ldo + o] = from_f<T>(a);
+}
+
+// block: keys a workgroup takes at a time (a multiple of 16 keeps a page's slots together; any value >= 1 is right).
+// partial: [rows * n_splits * H * VD] floats where n_splits > 1.
+TIS_EXPORT int tis_attention_mixed(int dtype, const void* q, long ldq, const void* plane, const int* block_tables, int bt_ld,
+                                   const int* row_seq, const int* positions, void* out, long ldo, float* partial,
+                                   int n_splits, int rows, int H, int G, int KD, int VD, int page_size, int chunk_size,
+                                   float scale, float softcap, const float* head_bias, const float* talk, int block,
+                                   hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || H < 1 || G < 1 || H % G || KD < 1 || VD < 1 || page_size < 1 || chunk_size < 0 || block < 1 ||
+      n_splits < 1 || n_splits > 65535 || !head_bias || !talk || softcap < 0.f)
+    return tis_fail("attention_mixed: bad size rows=%d heads=%d kv_heads=%d key=%d value=%d page=%d chunk=%d block=%d splits=%d",
+                    rows, H, G, KD, VD, page_size, chunk_size, block, n_splits);
+  if ((long)H * VD > (long)AM_PER * AW_THREADS)
+    return tis_fail("attention_mixed: %d heads of %d value channels are more than %d outputs a row", H, VD, AM_PER * AW_THREADS);
+  const long lds = ((long)H * KD + (long)H * H + 2L * H * block) * sizeof(float);
+  if (lds > 64 * 1024) return tis_fail("attention_mixed: %ld bytes of LDS for %d heads of %d in blocks of %d keys", lds, H, KD, block);
+  if (n_splits > 1 && !partial) return tis_fail("attention_mixed: key splits without a workspace");
+  dim3 grid(rows, n_splits);
+  const long merge_blocks = ((long)rows * H * VD + AW_THREADS - 1) / AW_THREADS;
+  if (dtype == TIS_F32) {
+    attention_mixed_kernel<float><<<grid, AW_THREADS, lds, stream>>>((const float*)q, ldq, (const float*)plane, block_tables,
+        bt_ld, row_seq, positions, (float*)out, ldo, partial, n_splits, H, G, KD, VD, page_size, chunk_size, scale, softcap,
+        head_bias, talk, block);
+    if (n_splits > 1)
+      attention_mixed_merge_kernel<float><<<merge_blocks, AW_THREADS, 0, stream>>>(partial, n_splits, (float*)out, ldo, rows, H * VD);
+  } else if (dtype == TIS_BF16) {
+    attention_mixed_kernel<bf16><<<grid, AW_THREADS, lds, stream>>>((const bf16*)q, ldq, (const bf16*)plane, block_tables,
+        bt_ld, row_seq, positions, (bf16*)out, ldo, partial, n_splits, H, G, KD, VD, page_size, chunk_size, scale, softcap,
+        head_bias, talk, block);
+    if (n_splits > 1)
+      attention_mixed_merge_kernel<bf16><<<merge_blocks, AW_THREADS, 0, stream>>>(partial, n_splits, (bf16*)out, ldo, rows, H * VD);
+  } else {
+    return tis_fail("unknown dtype code %d", dtype);
+  }
+  return tis_launch_status("attention_mixed");
+}

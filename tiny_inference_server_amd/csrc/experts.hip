@@ -30,7 +30,8 @@ __device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.f + 
 __global__ __launch_bounds__(TIS_WAVE) void route_topk_kernel(const float* __restrict__ z, long ldz,
                                                               const float* __restrict__ correction, float scale,
                                                               int n_out, int top, int score, int* __restrict__ ids,
-                                                              float* __restrict__ weights) {
+                                                              float* __restrict__ weights, int n_groups, int keep,
+                                                              int renorm) {
   const long r = blockIdx.x;
   const int lane = threadIdx.x;
   float s[EX_MAX_PER_LANE], c[EX_MAX_PER_LANE];
@@ -58,13 +59,43 @@ __global__ __launch_bounds__(TIS_WAVE) void route_topk_kernel(const float* __res
     s[u] *= inv;
     c[u] = e < n_out ? s[u] + (correction ? correction[e] : 0.f) : -INFINITY;
   }
+  if (n_groups > 1 && keep < n_groups) {
+    // The outputs form n_groups equal runs of neighbours; a group's score is its largest c. Only outputs of the `keep`
+    // best groups (the lower group keeps a tie) stay in the choice; the others' c become -inf. Up to 64 groups: lane g
+    // holds group g's score.
+    const int per = n_out / n_groups;
+    float gs = -INFINITY;
+    for (int g = 0; g < n_groups; ++g) {
+      float m = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
+        const int e = lane + u * TIS_WAVE;
+        if (e < n_out && e / per == g) m = fmaxf(m, c[u]);
+      }
+      m = wave_max(m);
+      if (lane == g) gs = m;
+    }
+    // a group's rank: how many groups beat it
+    int rank = 0;
+    for (int g = 0; g < n_groups; ++g) {
+      const float og = __shfl(gs, g, TIS_WAVE);
+      if (og > gs || (og == gs && g < lane)) ++rank;
+    }
+    const unsigned long long kept = __ballot(lane < n_groups && rank < keep);
+#pragma unroll
+    for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
+      const int e = lane + u * TIS_WAVE;
+      if (e < n_out && !((kept >> (e / per)) & 1ull)) c[u] = -INFINITY;
+    }
+  }
+  float total = 0.f;
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY;
     int at = 0x7fffffff;
 #pragma unroll
     for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
       const int e = lane + u * TIS_WAVE;
-      if (c[u] > best) { best = c[u]; at = e; }       // rising e within a lane: the lower index keeps a tie
+      if (e < n_out && c[u] > best) { best = c[u]; at = e; }       // rising e within a lane: the lower index keeps a tie
     }
 #pragma unroll
     for (int o = TIS_WAVE / 2; o > 0; o >>= 1) {
@@ -78,10 +109,16 @@ __global__ __launch_bounds__(TIS_WAVE) void route_topk_kernel(const float* __res
       if (lane + u * TIS_WAVE == at) { w = s[u]; c[u] = -INFINITY; }
     }
     w = wave_sum(w);          // only the owner's lane holds it
+    total += w;
     if (lane == 0) {
       ids[r * top + k] = at;
       weights[r * top + k] = w * scale;
     }
+  }
+  // renorm: the chosen weights divided by their sum (lane 0 reads back what it wrote itself)
+  if (renorm && lane == 0) {
+    const float inv = 1.f / (total + 1e-20f);
+    for (int k = 0; k < top; ++k) weights[r * top + k] *= inv;
   }
 }
 
@@ -371,12 +408,14 @@ __global__ __launch_bounds__(256) void experts_combine_kernel(const float* __res
 }
 
 TIS_EXPORT int tis_route_topk(const float* z, long ldz, const float* correction, float scale, int rows, int n_out, int top, int score,
-                              int* ids, float* weights, hipStream_t stream) {
+                              int* ids, float* weights, int n_groups, int keep, int renorm, hipStream_t stream) {
   if (rows == 0) return 0;
+  if (n_groups < 1 || n_groups > TIS_WAVE || n_out % n_groups || keep < 1 || keep > n_groups || top > keep * (n_out / n_groups))
+    return tis_fail("route_topk: %d outputs in %d groups (at most %d) of which %d are kept, top %d", n_out, n_groups, TIS_WAVE, keep, top);
   if (rows < 0 || n_out < 1 || n_out > EX_MAX_PER_LANE * TIS_WAVE || top < 1 || top > n_out)
     return tis_fail("route_topk: bad size rows=%d outputs=%d (at most %d) top=%d", rows, n_out, EX_MAX_PER_LANE * TIS_WAVE, top);
   if (score != 0 && score != 1) return tis_fail("route_topk: score kind %d (0: softmax, 1: sigmoid)", score);
-  route_topk_kernel<<<rows, TIS_WAVE, 0, stream>>>(z, ldz, correction, scale, n_out, top, score, ids, weights);
+  route_topk_kernel<<<rows, TIS_WAVE, 0, stream>>>(z, ldz, correction, scale, n_out, top, score, ids, weights, n_groups, keep, renorm);
   return tis_launch_status("route_topk");
 }
 

@@ -171,6 +171,10 @@ struct ChosenSum {
   int top, n_experts;
   const void* rows;      // [rows][ldr] in the compute type: what the feed-forward read
   long ldr;
+  const float* extra = nullptr;        // [rows][lde]: what every row adds beside its choices (a shared expert's result),
+  long lde = 0;                        // times sigmoid(extra_gate[row * ldg]); null: nothing
+  const float* extra_gate = nullptr;
+  long ldg = 0;
 };
 
 // PER: values a thread keeps in registers (width <= 256 * PER), so that the row is read once and the sums follow one
@@ -203,6 +207,7 @@ __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
       const float w = kept ? chosen_w[k] : cs.weights[r * cs.top + k];
       v += w * (e < cs.n_experts ? y_in[(r * cs.top + k) * ldy + c] : to_f(static_cast<const T*>(cs.rows)[r * cs.ldr + c]));
     }
+    if (cs.extra) v += sigmoid_f(cs.extra_gate[r * cs.ldg]) * cs.extra[r * cs.lde + c];
     return v;
   };
   // (everything the row's columns need is asked for at once: the gains and the bias too, which are only used after
@@ -395,12 +400,14 @@ TIS_EXPORT int tis_layernorm32(int dtype, const float* x, const float* gain, con
 TIS_EXPORT int tis_residual_norm(int dtype, const float* x, const float* y, long ldy, const float* y_gain, float y_eps,
                                  float* out32, void* copy, long ldc, int norm_kind, const float* gain, const float* bias,
                                  float eps, void* normed, long ldn, int rows, int D, const int* ids, const float* weights,
-                                 int top, int n_experts, const void* chosen_rows, long ldr, hipStream_t stream) {
+                                 int top, int n_experts, const void* chosen_rows, long ldr, const float* extra, long lde,
+                                 const float* extra_gate, long ldg, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || D < 1 || !x || !out32) return tis_fail("residual_norm: bad arguments rows=%d width=%d", rows, D);
   if (ids && (!weights || top < 1 || n_experts < 0 || (n_experts > 0 && !y) || !chosen_rows))
     return tis_fail("residual_norm: a sum over chosen experts needs ids, weights, the experts' results and the rows they read");
-  const ChosenSum cs{ids, weights, top, n_experts, chosen_rows, ldr};
+  if (extra && (!ids || !extra_gate)) return tis_fail("residual_norm: a shared term goes with chosen experts and has a gate");
+  const ChosenSum cs{ids, weights, top, n_experts, chosen_rows, ldr, extra, lde, extra_gate, ldg};
   if (norm_kind < 0 || norm_kind > 2 || (norm_kind && (!gain || !normed)))
     return tis_fail("residual_norm: norm kind %d needs a gain and an output", norm_kind);
 #define S32_RESIDUAL(T, PER)                                                                                              \
@@ -512,13 +519,19 @@ template <typename T>
 __global__ __launch_bounds__(S32_THREADS) void gated_act_kernel(const float* __restrict__ z, long ldz, int F,
                                                                  const float* __restrict__ gb, const float* __restrict__ ub,
                                                                  const float* __restrict__ row_scale, int act,
-                                                                 T* __restrict__ out, long ldo, int rows) {
+                                                                 T* __restrict__ out, long ldo, int rows, float limit) {
   const long i = (long)blockIdx.x * S32_THREADS + threadIdx.x;
   if (i >= (long)rows * F) return;
   const long r = i / F;
   const int j = (int)(i % F);
   const float w = row_scale ? row_scale[r] : 1.f;
-  const float g = w * (z[r * ldz + j] + (gb ? gb[j] : 0.f)), u = w * (z[r * ldz + F + j] + (ub ? ub[j] : 0.f));
+  float g = w * (z[r * ldz + j] + (gb ? gb[j] : 0.f)), u = w * (z[r * ldz + F + j] + (ub ? ub[j] : 0.f));
+  if (act == 2) {      // g sigmoid(1.702 g) (u + 1) with g capped from above and u from both sides at `limit`
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    out[r * ldo + j] = from_f<T>(g * sigmoid_f(1.702f * g) * (u + 1.f));
+    return;
+  }
   out[r * ldo + j] = from_f<T>((act == 0 ? gelu_tanh_f(g) : g * sigmoid_f(g)) * u);
 }
 
@@ -563,12 +576,13 @@ TIS_EXPORT int tis_scaled_sum(int dtype, const float* x, const float* y0, long l
 }
 
 TIS_EXPORT int tis_gated_act(int dtype, const float* z, long ldz, int F, const float* gate_bias, const float* up_bias,
-                             const float* row_scale, int act, void* out, long ldo, int rows, hipStream_t stream) {
+                             const float* row_scale, int act, void* out, long ldo, int rows, float limit, hipStream_t stream) {
   if (rows == 0) return 0;
-  if (rows < 0 || F < 1 || (act != 0 && act != 1)) return tis_fail("gated_act: bad size rows=%d hidden=%d act=%d", rows, F, act);
+  if (rows < 0 || F < 1 || act < 0 || act > 2 || (act == 2 && !(limit > 0.f)))
+    return tis_fail("gated_act: bad size rows=%d hidden=%d act=%d limit=%g", rows, F, act, (double)limit);
   const long blocks = ((long)rows * F + S32_THREADS - 1) / S32_THREADS;
-  S32_DISPATCH((gated_act_kernel<float><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, F, gate_bias, up_bias, row_scale, act, (float*)out, ldo, rows)),
-               (gated_act_kernel<bf16><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, F, gate_bias, up_bias, row_scale, act, (bf16*)out, ldo, rows)))
+  S32_DISPATCH((gated_act_kernel<float><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, F, gate_bias, up_bias, row_scale, act, (float*)out, ldo, rows, limit)),
+               (gated_act_kernel<bf16><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, F, gate_bias, up_bias, row_scale, act, (bf16*)out, ldo, rows, limit)))
   return tis_launch_status("gated_act");
 }
 
@@ -578,4 +592,101 @@ TIS_EXPORT int tis_softcap(float* z, long ldz, float cap, int rows, int W, hipSt
   const long blocks = ((long)rows * W + S32_THREADS - 1) / S32_THREADS;
   softcap_kernel<<<blocks, S32_THREADS, 0, stream>>>(z, ldz, cap, rows, W);
   return tis_launch_status("softcap");
+}
+
+// ---- blocks with a norm on both sides of a sublayer, several mixers side by side -----------------------------------
+
+// out[r][c] = act(z) with z = sum_k low[r][k] * w2[c][k] + bias[c] (bias may be null): the second half of a low-rank
+// projection, in 32-bit. kind 0: sigmoid(z)^(1/tau); 1: exp(-rate[c / group] * softplus(z)), a decay whose rate is one
+// number per run of `group` channels; 2: z itself.
+__global__ __launch_bounds__(S32_THREADS) void lowrank_act_kernel(const float* __restrict__ low, long ldl, int rank,
+                                                                   const float* __restrict__ w2,
+                                                                   const float* __restrict__ bias, int kind, float tau,
+                                                                   const float* __restrict__ rate, int group,
+                                                                   float* __restrict__ out, int C, int row_blocks) {
+  extern __shared__ float a[];
+  const long r = blockIdx.x / row_blocks;        // a row's blocks of channels side by side: a few rows still fill the chip
+  for (int k = threadIdx.x; k < rank; k += S32_THREADS) a[k] = low[r * ldl + k];
+  __syncthreads();
+  const int c = (blockIdx.x % row_blocks) * S32_THREADS + threadIdx.x;
+  if (c >= C) return;
+  float z = 0.f;
+  const float* w = w2 + (long)c * rank;
+  for (int k = 0; k < rank; ++k) z += a[k] * w[k];
+  if (bias) z += bias[c];
+  if (kind == 0) z = expf(log_sigmoid_f(z) / tau);
+  else if (kind == 1) z = expf(-rate[c / group] * (z > 20.f ? z : log1pf(expf(z))));
+  out[r * C + c] = z;
+}
+
+// out[r] = (1 / n) * sum_i y_i[r] / sqrt(mean(y_i[r]^2) + eps) * gain_i: the mean of one or two RMS-normed rows, 32-bit.
+// One workgroup a row; the sums' order depends on the width alone.
+__global__ __launch_bounds__(S32_THREADS) void normed_mean_kernel(const float* __restrict__ y0, long ld0,
+                                                                   const float* __restrict__ g0,
+                                                                   const float* __restrict__ y1, long ld1,
+                                                                   const float* __restrict__ g1, float eps,
+                                                                   float* __restrict__ out, int D) {
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  float s0 = 0.f, s1 = 0.f;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    const float a = y0[r * ld0 + c];
+    s0 += a * a;
+    if (y1) {
+      const float b = y1[r * ld1 + c];
+      s1 += b * b;
+    }
+  }
+  const float i0 = 1.f / sqrtf(block_sum(s0, red) / (float)D + eps);
+  const float i1 = y1 ? 1.f / sqrtf(block_sum(s1, red) / (float)D + eps) : 0.f;
+  const float share = y1 ? 0.5f : 1.f;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    float v = y0[r * ld0 + c] * i0 * g0[c];
+    if (y1) v += y1[r * ld1 + c] * i1 * g1[c];
+    out[r * D + c] = v * share;
+  }
+}
+
+// out = act(z) in the compute type, z 32-bit (a strided view is fine). act 0: tanh-form gelu, 1: silu, 2: sigmoid,
+// 3: the square of relu.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void activate_rows_kernel(const float* __restrict__ z, long ldz, int act,
+                                                                     T* __restrict__ out, long ldo, int rows, int W) {
+  const long i = (long)blockIdx.x * S32_THREADS + threadIdx.x;
+  if (i >= (long)rows * W) return;
+  const long r = i / W;
+  const int j = (int)(i % W);
+  const float v = z[r * ldz + j];
+  const float p = fmaxf(v, 0.f);
+  out[r * ldo + j] = from_f<T>(act == 0 ? gelu_tanh_f(v) : act == 1 ? v * sigmoid_f(v) : act == 2 ? sigmoid_f(v) : p * p);
+}
+
+TIS_EXPORT int tis_lowrank_act(const float* low, long ldl, int rank, const float* w2, const float* bias, int kind, float tau,
+                               const float* rate, int group, float* out, int rows, int C, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || rank < 1 || rank > 8192 || C < 1 || kind < 0 || kind > 2 || (kind == 0 && !(tau > 0.f)) ||
+      (kind == 1 && (!rate || group < 1)))
+    return tis_fail("lowrank_act: bad arguments rows=%d rank=%d channels=%d kind=%d", rows, rank, C, kind);
+  const int row_blocks = (C + S32_THREADS - 1) / S32_THREADS;
+  lowrank_act_kernel<<<(long)rows * row_blocks, S32_THREADS, rank * sizeof(float), stream>>>(low, ldl, rank, w2, bias, kind, tau,
+                                                                                            rate, group, out, C, row_blocks);
+  return tis_launch_status("lowrank_act");
+}
+
+TIS_EXPORT int tis_normed_mean(const float* y0, long ld0, const float* g0, const float* y1, long ld1, const float* g1, float eps,
+                               float* out, int rows, int D, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1 || !y0 || !g0 || (y1 && !g1) || !out) return tis_fail("normed_mean: bad arguments rows=%d width=%d", rows, D);
+  normed_mean_kernel<<<rows, S32_THREADS, 0, stream>>>(y0, ld0, g0, y1, ld1, g1, eps, out, D);
+  return tis_launch_status("normed_mean");
+}
+
+TIS_EXPORT int tis_activate_rows(int dtype, const float* z, long ldz, int act, void* out, long ldo, int rows, int W,
+                                 hipStream_t stream) {
+  if (rows == 0 || W == 0) return 0;
+  if (rows < 0 || W < 0 || act < 0 || act > 3) return tis_fail("activate_rows: bad size rows=%d width=%d act=%d", rows, W, act);
+  const long blocks = ((long)rows * W + S32_THREADS - 1) / S32_THREADS;
+  S32_DISPATCH((activate_rows_kernel<float><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, act, (float*)out, ldo, rows, W)),
+               (activate_rows_kernel<bf16><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, act, (bf16*)out, ldo, rows, W)))
+  return tis_launch_status("activate_rows");
 }

@@ -46,6 +46,7 @@ SOURCES: Dict[str, str] = {
     "experts": "experts.hip",
     "attention_latent": "attention_latent.hip",
     "ssm_parts": "ssm_parts.hip",
+    "delta_rule": "delta_rule.hip",
 }
 HEADERS = ["common.h", "attention_mfma.h"]
 # what a library links beyond the HIP runtime

@@ -110,27 +110,32 @@ _SIGNATURES["stream32"] = ("tis_stream32", {
     "tis_head_norm_gate": [_I, _P, _L, _P, _L, _P, _I, _I, _F, _P, _L, _I, _I, _I, _P],
     "tis_lowrank_decay": [_P, _L, _I, _P, _P, _F, _P, _I, _I, _P],
     "tis_layernorm32": [_I, _P, _P, _P, _F, _P, _L, _I, _I, _P],
-    "tis_residual_norm": [_I, _P, _P, _L, _P, _F, _P, _P, _L, _I, _P, _P, _F, _P, _L, _I, _I, _P, _P, _I, _I, _P, _L, _P],
+    "tis_residual_norm": [_I, _P, _P, _L, _P, _F, _P, _P, _L, _I, _P, _P, _F, _P, _L, _I, _I, _P, _P, _I, _I, _P, _L, _P, _L,
+                          _P, _L, _P],
     "tis_gate_table": [_I, _P, _L, _P, _L, _P, _I, _P, _L, _I, _I, _P],
     "tis_activate32": [_P, _L, _I, _I, _I, _P],
     "tis_head_gate": [_I, _P, _L, _P, _L, _I, _I, _I, _P],
     "tis_dyt32": [_I, _P, _F, _P, _P, _P, _L, _I, _I, _P],
     "tis_scaled_sum": [_I, _P, _P, _L, _P, _P, _P, _L, _P, _P, _P, _P, _I, _I, _P, _L, _P, _I, _F, _P, _P, _P, _L, _I, _I,
                        _P],
-    "tis_gated_act": [_I, _P, _L, _I, _P, _P, _P, _I, _P, _L, _I, _P],
+    "tis_gated_act": [_I, _P, _L, _I, _P, _P, _P, _I, _P, _L, _I, _F, _P],
     "tis_softcap": [_P, _L, _F, _I, _I, _P],
+    "tis_lowrank_act": [_P, _L, _I, _P, _P, _I, _F, _P, _I, _P, _I, _I, _P],
+    "tis_normed_mean": [_P, _L, _P, _P, _L, _P, _F, _P, _I, _I, _P],
+    "tis_activate_rows": [_I, _P, _L, _I, _P, _L, _I, _I, _P],
 })
 _SIGNATURES["attention_window"] = ("tis_attention_window", {
     "tis_attention_prepare": [_I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _F, _I,
                               _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "tis_latent_prepare": [_I, _P, _L, _I, _I, _P, _P, _P, _P, _L, _P, _L, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P],
     "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _P],
+    "tis_attention_mixed": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P, _P, _I, _P],
 })
 _SIGNATURES["attention_latent"] = ("tis_attention_latent", {
     "tis_attention_latent": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
 })
 _SIGNATURES["experts"] = ("tis_experts", {
-    "tis_route_topk": [_P, _L, _P, _F, _I, _I, _I, _I, _P, _P, _P],
+    "tis_route_topk": [_P, _L, _P, _F, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P],
     "tis_expert_lists": [_P, _I, _I, _I, _P, _P, _P],
     "tis_grouped_linear": [_I, _I, _P, _L, _L, _I, _P, _P, _L, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "tis_experts_combine": [_I, _P, _L, _P, _L, _P, _P, _I, _I, _P, _L, _I, _I, _P],
@@ -143,6 +148,11 @@ _SIGNATURES["ssm_parts"] = ("tis_ssm", {
     "tis_conv_prepare": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _L, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P],
     "tis_conv_state_update": [_P, _L, _I, _P, _L, _I, _P, _P, _I, _I, _I, _P],
     "tis_gated_group_norm": [_I, _P, _L, _P, _L, _P, _I, _P, _L, _P, _F, _P, _L, _I, _I, _I, _P],
+})
+
+_SIGNATURES["delta_rule"] = ("tis_delta_rule", {
+    "tis_delta_prepare": [_P, _L, _I, _I, _P, _I, _P, _L, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P],
+    "tis_delta_scan": [_P, _L, _I, _I, _I, _I, _P, _L, _P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _I, _P],
 })
 
 _libs = {}
@@ -1239,6 +1249,9 @@ class HipOps:
                                   f"{tuple(chosen.rows.shape)} for {n} rows of {D} with {top} choices")
             if y is not None:
                 self._f32_rows(y, "experts' results", n * top, D)
+            if chosen.extra is not None:
+                self._f32_rows(chosen.extra, "what every row adds beside its choices", n, D)
+                self._f32_rows(chosen.extra_gate, "that term's gate", n, 1)
         elif y is not None:
             self._f32_rows(y, "residual_norm y", n, D)
         elif y_rms is not None:
@@ -1255,13 +1268,16 @@ class HipOps:
         as_is = self.dtype == torch.float32
         cp = self.empty(n, D) if copy and not as_is else None
         normed = self.empty(n, D) if kind else None
+        extra = chosen.extra if chosen is not None else None
         self._lazy("stream32").tis_residual_norm(
             self.code, _ptr(x32), _ptr(y), y.stride(0) if y is not None else 0, _ptr(y_rms[0] if y_rms else None),
             float(y_rms[1]) if y_rms else 0.0, _ptr(x32), _ptr(cp), cp.stride(0) if cp is not None else 0, kind, _ptr(gain),
             _ptr(bias), float(eps), _ptr(normed), normed.stride(0) if normed is not None else 0, n, D,
             _ptr(chosen.ids if chosen else None), _ptr(chosen.weights if chosen else None),
             chosen.ids.shape[1] if chosen else 0, chosen.n_experts if chosen else 0,
-            _ptr(chosen.rows if chosen else None), chosen.rows.stride(0) if chosen else 0, self._stream())
+            _ptr(chosen.rows if chosen else None), chosen.rows.stride(0) if chosen else 0,
+            _ptr(extra), extra.stride(0) if extra is not None else 0, _ptr(chosen.extra_gate if extra is not None else None),
+            chosen.extra_gate.stride(0) if extra is not None else 0, self._stream())
         return x32, (x32 if copy and as_is else cp), normed
 
     _ACTS = {"gelu_tanh": 0, "silu": 1, "sigmoid": 2}
@@ -1361,11 +1377,12 @@ class HipOps:
             normed.stride(0) if normed is not None else 0, n, D, self._stream())
         return x32, normed
 
-    _GATED_ACTS = {"gelu_tanh": 0, "silu": 1}
+    _GATED_ACTS = {"gelu_tanh": 0, "silu": 1, "clamped_swish": 2}
 
-    def gated_act(self, z, hidden: int, act: str, gate_bias=None, up_bias=None, row_scale=None):
+    def gated_act(self, z, hidden: int, act: str, gate_bias=None, up_bias=None, row_scale=None, limit: float = 0.0):
         """act(w * (z[:, :hidden] + gate_bias)) * (w * (z[:, hidden:2 hidden] + up_bias)) in the compute type, w being
-        row_scale [rows] (None: 1). z: [rows, >= 2 hidden] 32-bit (a strided view is fine); act: "gelu_tanh" or "silu"."""
+        row_scale [rows] (None: 1). z: [rows, >= 2 hidden] 32-bit (a strided view is fine); act: "gelu_tanh", "silu", or
+        "clamped_swish": g sigmoid(1.702 g) (u + 1) with g = min(gate, limit) and u = clamp(up, -limit, limit)."""
         n = z.shape[0]
         self._f32_rows(z, "gated_act z", n, 2 * hidden)
         for t, what, size in ((gate_bias, "gate bias", hidden), (up_bias, "up bias", hidden), (row_scale, "row factors", n)):
@@ -1376,7 +1393,60 @@ class HipOps:
         out = self.empty(n, hidden)
         self._lazy("stream32").tis_gated_act(self.code, _ptr(z), z.stride(0), int(hidden), _ptr(gate_bias), _ptr(up_bias),
                                              _ptr(row_scale), self._GATED_ACTS[act], _ptr(out), out.stride(0), n,
-                                             self._stream())
+                                             float(limit), self._stream())
+        return out
+
+    _ROW_ACTS = {"gelu_tanh": 0, "silu": 1, "sigmoid": 2, "relu2": 3}
+
+    def activate_rows(self, z, act: str):
+        """act(z) in the compute type. z: [rows, W] 32-bit (a strided view is fine); act: "gelu_tanh", "silu", "sigmoid"
+        or "relu2" (the square of relu)."""
+        _rows_view(self._check(z, "activate_rows z", torch.float32), "activate_rows z")
+        if act not in self._ROW_ACTS:
+            raise KernelError(f"activate_rows: activation {act!r} (known: {', '.join(self._ROW_ACTS)})")
+        n, W = z.shape
+        out = self.empty(n, W)
+        self._lazy("stream32").tis_activate_rows(self.code, _ptr(z), z.stride(0), self._ROW_ACTS[act], _ptr(out), out.stride(0),
+                                                 n, W, self._stream())
+        return out
+
+    def normed_mean(self, branches, eps: float):
+        """The mean of one or two rows after an RMS norm each: (1 / n) sum_i y_i / sqrt(mean(y_i^2) + eps) * gain_i, in
+        32-bit. branches: (y [rows, width] 32-bit (a strided view is fine), gain [width])."""
+        if not 1 <= len(branches) <= 2:
+            raise KernelError(f"normed_mean: {len(branches)} branches (one or two)")
+        n, D = branches[0][0].shape
+        for y, gain in branches:
+            self._f32_rows(y, "normed_mean branch", n, D)
+            self._f32(gain, "normed_mean gain", D)
+        (y0, g0), (y1, g1) = branches[0], (branches[1] if len(branches) > 1 else (None, None))
+        out = torch.empty(n, D, dtype=torch.float32, device=self.device)
+        self._lazy("stream32").tis_normed_mean(_ptr(y0), y0.stride(0), _ptr(g0), _ptr(y1), y1.stride(0) if y1 is not None else 0,
+                                               _ptr(g1), float(eps), _ptr(out), n, D, self._stream())
+        return out
+
+    _LOWRANK_KINDS = {"sigmoid_root": 0, "exp_softplus": 1, "none": 2}
+
+    def lowrank_act(self, low, w2, bias, kind: str, rate=None, group: int = 1, tau: float = 1.0):
+        """The second half of a low-rank projection in 32-bit: act(low . w2^T + bias) with low [rows, rank] (a strided view
+        is fine), w2 [channels, rank], bias [channels] or None. kind "sigmoid_root": sigmoid(z)^(1/tau); "exp_softplus":
+        exp(-rate[c // group] * softplus(z)), a decay with one rate per run of `group` channels; "none": z."""
+        n, rank = low.shape
+        _rows_view(self._check(low, "lowrank_act low", torch.float32), "lowrank_act low")
+        C = w2.shape[0]
+        self._f32(w2, "lowrank_act w2", C * rank)
+        if bias is not None:
+            self._f32(bias, "lowrank_act bias", C)
+        if kind not in self._LOWRANK_KINDS:
+            raise KernelError(f"lowrank_act: kind {kind!r} (known: {', '.join(self._LOWRANK_KINDS)})")
+        if kind == "exp_softplus":
+            if group < 1 or C % group:
+                raise KernelError(f"lowrank_act: {C} channels in runs of {group}")
+            self._f32(rate, "lowrank_act rates", C // group)
+        out = torch.empty(n, C, dtype=torch.float32, device=self.device)
+        self._lazy("stream32").tis_lowrank_act(_ptr(low), low.stride(0), rank, _ptr(w2), _ptr(bias), self._LOWRANK_KINDS[kind],
+                                               float(tau), _ptr(rate if kind == "exp_softplus" else None), int(group),
+                                               _ptr(out), n, C, self._stream())
         return out
 
     def softcap(self, z, cap: float):
@@ -1485,10 +1555,12 @@ class HipOps:
             self._grouped(x, x.stride(0), K, 1, w, out[:, out_offset:], out.stride(0), out_group, None, None, 0, n)
         return out
 
-    def route_topk(self, z, correction, scale: float, top: int, score: str = "softmax"):
+    def route_topk(self, z, correction, scale: float, top: int, score: str = "softmax", groups=None, renorm: bool = False):
         """A router's choice: (ids [rows, top] int32, weights [rows, top] 32-bit). s = softmax(z) over a row's outputs
         (score "sigmoid": sigmoid(z), each output by itself); the `top` outputs with the largest s + correction are
-        chosen; an output's weight is s * scale."""
+        chosen; an output's weight is s * scale. groups = (count, keep): the outputs form `count` equal runs of
+        neighbours, a group's score is its largest s + correction, and only outputs of the `keep` best groups can be
+        chosen. renorm: the chosen weights are divided by their sum (+ 1e-20) before the scale."""
         if score not in ("softmax", "sigmoid"):
             raise KernelError(f"route_topk: score {score!r} (known: 'softmax', 'sigmoid')")
         n, E = z.shape
@@ -1497,8 +1569,12 @@ class HipOps:
             self._f32(correction, "router correction", E)
         ids = torch.empty(n, top, dtype=torch.int32, device=self.device)
         weights = torch.empty(n, top, dtype=torch.float32, device=self.device)
+        count, keep = (int(groups[0]), int(groups[1])) if groups is not None else (1, 1)
+        if count < 1 or E % count or not 1 <= keep <= count or top > keep * (E // count):
+            raise KernelError(f"route_topk: {E} outputs in {count} groups of which {keep} are kept, top {top}")
         self._lazy("experts").tis_route_topk(_ptr(z), z.stride(0), _ptr(correction), float(scale), n, E, int(top),
-                                             1 if score == "sigmoid" else 0, _ptr(ids), _ptr(weights), self._stream())
+                                             1 if score == "sigmoid" else 0, _ptr(ids), _ptr(weights), count, keep,
+                                             1 if renorm else 0, self._stream())
         return ids, weights
 
     def routed_experts(self, x, ids, weights, w_up, w_down, act: str = "gelu_erf", combine: bool = True):
@@ -1534,7 +1610,8 @@ class HipOps:
                                 n, D, self._stream())
         return out
 
-    def gated_experts(self, x, ids, weights, w_gate_up, w_down, act: str = "silu"):
+    def gated_experts(self, x, ids, weights, w_gate_up, w_down, act: str = "silu", limit: float = 0.0, weigh: str = "input",
+                      n_experts=None):
         """Gated experts whose router weight scales the expert's input: for every (row, choice) the line
         w_down[e] . (act(w * g) * (w * u)) with [g | u] = w_gate_up[e] . x, e = ids[row, choice], w = weights[row,
         choice] (an expert without biases applied to w * x), in 32-bit, not summed: a `ChosenExperts` whose weights are
@@ -1543,13 +1620,31 @@ class HipOps:
         _rows_view(self._check(x, "experts x"), "experts x")
         n, D = x.shape
         top = ids.shape[1]
-        E, F2 = w_gate_up.shape[0], w_gate_up.shape[1]
-        F = F2 // 2
         self._index(ids, "expert ids", n * top)
         self._f32(weights, "expert weights", n * top)
+        if weigh not in ("input", "output"):
+            raise KernelError(f"gated_experts: weigh {weigh!r} ('input' or 'output')")
+        # weigh "output": a chosen expert's weight multiplies its result (in the sum over a row's choices, which the
+        # residual sum takes); ids from the number of matrices on are identity experts whose result is the row itself
+        if w_gate_up is None:
+            if weigh != "output":
+                raise KernelError("gated_experts: identity experts alone weigh their results")
+            return ChosenExperts(None, ids, weights, 0, x)
+        E, F2 = w_gate_up.shape[0], w_gate_up.shape[1]
+        F = F2 // 2
         if E < 1 or F2 % 2 or tuple(w_gate_up.shape) != (E, 2 * F, D) or tuple(w_down.shape) != (E, D, F):
             raise KernelError(f"gated_experts: matrices {tuple(w_gate_up.shape)} and {tuple(w_down.shape)} for width {D}")
         y = torch.empty(n * top, D, dtype=torch.float32, device=self.device)
+        if weigh == "output":
+            if n:
+                lists = torch.empty(E, n, dtype=torch.int32, device=self.device)
+                counts = torch.empty(E, dtype=torch.int32, device=self.device)
+                self._lazy("experts").tis_expert_lists(_ptr(ids), n * top, E, n, _ptr(lists), _ptr(counts), self._stream())
+                z = torch.empty(n * top, 2 * F, dtype=torch.float32, device=self.device)
+                self._grouped(x, x.stride(0), 0, top, w_gate_up, z, z.stride(0), 0, lists, counts, n, n)
+                hidden = self.gated_act(z, F, act, limit=limit)
+                self._grouped(hidden, hidden.stride(0), 0, 1, w_down, y, D, 0, lists, counts, n, n)
+            return ChosenExperts(y, ids, weights, E, x)
         if n:
             lists = torch.empty(E, n, dtype=torch.int32, device=self.device)
             counts = torch.empty(E, dtype=torch.int32, device=self.device)
@@ -1559,6 +1654,11 @@ class HipOps:
             hidden = self.gated_act(z, F, act, row_scale=weights.view(-1))
             self._grouped(hidden, hidden.stride(0), 0, 1, w_down, y, D, 0, lists, counts, n, n)
         return ChosenExperts(y, ids, None, E, x)
+
+    def combine_experts(self, chosen):
+        """The sum that a `ChosenExperts` stands for, as 32-bit rows (a block's residual sum usually takes it instead)."""
+        n, D = chosen.rows.shape
+        return self.residual_norm(torch.zeros(n, D, dtype=torch.float32, device=self.device), chosen)[0]
 
     # ---- attention with keys and values of different sizes -----------------------------------------------
     def _check_kv_plane(self, plane, n_kv_heads, key_dim, value_dim, page_size):
@@ -1722,6 +1822,100 @@ class HipOps:
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, key_dim, value_dim, page_size,
             int(window), int(chunk), float(scale if scale is not None else key_dim ** -0.5), 1 if sink else 0, _ptr(gate),
             gate.stride(0) if gate is not None else 0, self._stream())
+        return out
+
+    def mixed_sigmoid_attention(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, chunk,
+                                scale, softcap, head_bias, talk):
+        """Attention of the rows in `batch` whose weights are sigmoids mixed across the heads: for every key j that the
+        row at position p sees (j <= p; chunk > 0: only from p - p % chunk on), w_g = sigmoid(cap(q_g . k * scale) +
+        head_bias[g]) with cap(s) = softcap * tanh(s / softcap) (softcap 0: s), head h weighs the values of its own
+        key/value head with sum_g talk[h, g] * w_g. Nothing is normalised over the keys. [rows, heads * value_dim]."""
+        _rows_view(self._check(q, "q"), "q")
+        n = q.shape[0]
+        self._check_kv_plane(plane, n_kv_heads, key_dim, value_dim, page_size)
+        if q.shape[1] != n_heads * key_dim:
+            raise KernelError(f"attention: q width {q.shape[1]} is not heads {n_heads} x key size {key_dim}")
+        self._f32(head_bias, "attention head bias", n_heads)
+        self._f32(talk, "attention head mixture", n_heads * n_heads)
+        tables = batch.block_tables[group]
+        self._check(tables, "block tables", torch.int32)
+        if tables.dim() != 2 or tables.stride(1) != 1:
+            raise KernelError(f"attention: block tables {tuple(tables.shape)} must be 2-d")
+        self._index(batch.positions, "positions", n)
+        self._index(batch.row_seq, "row_seq", n)
+        if batch.max_kv_len > tables.shape[1] * page_size:
+            raise KernelError(f"attention: a row sees {batch.max_kv_len} keys but block tables cover "
+                              f"{tables.shape[1] * page_size}")
+        out = self.empty(n, n_heads * value_dim)
+        if n == 0:
+            return out
+        # keys a workgroup takes at a time: what LDS holds beside the row's queries, in whole pages
+        room = (16384 - n_heads * key_dim - n_heads * n_heads) // (2 * n_heads)
+        block = min(256, room // 16 * 16 if room >= 16 else room)
+        if block < 1:
+            raise KernelError(f"attention: {n_heads} heads of {key_dim} channels do not fit the kernel for any sizes")
+        # few rows: a row's keys are cut over several workgroups, whose parts a second kernel adds up
+        longest = min(batch.max_kv_len, chunk) if chunk > 0 else batch.max_kv_len
+        n_splits = int(max(1, min(-(-longest // block), (2 * self.units) // n, 64)))
+        partial = None
+        if n_splits > 1:
+            need = n * n_splits * n_heads * value_dim
+            partial = self._workspace if self._workspace.numel() >= need else torch.empty(need, dtype=torch.float32,
+                                                                                         device=self.device)
+        self._lazy("attention_window").tis_attention_mixed(
+            self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
+            _ptr(batch.positions), _ptr(out), out.stride(0), _ptr(partial), n_splits, n, n_heads, n_kv_heads, key_dim,
+            value_dim, page_size, int(chunk), float(scale), float(softcap), _ptr(head_bias), _ptr(talk), int(block),
+            self._stream())
+        return out
+
+    # ---- a gated delta rule ----------------------------------------------------------------------------------
+    def _check_lines(self, what, state, floats, batch):
+        self._check(state, "state", torch.float32)
+        if state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < floats:
+            raise KernelError(f"{what}: state {tuple(state.shape)} for lines of {floats} floats")
+        self._index(batch.cu_rows, "cu_rows", batch.n_seqs + 1)
+        self._index(batch.seq_slots, "seq_slots", batch.n_seqs)
+        if max(batch.host_slots, default=0) >= state.shape[0]:
+            raise KernelError(f"{what}: slot {max(batch.host_slots)} of {state.shape[0]}")
+
+    def delta_prepare(self, proj, conv_off, beta_off, taps, state, conv_at, batch, n_heads, qk_heads, dim, vdim):
+        """The step before a delta rule's walk, from a row's 32-bit projections: the columns conv_off.. hold q and k
+        (qk_heads * dim each) and v (heads * vdim), which go channel by channel through a short causal convolution
+        (taps [channels, taps], the last column weighs the row itself; earlier inputs come from the step's rows and
+        before those from the request's state line, from float conv_at on, [taps - 1][channels], oldest first) and silu;
+        q and k become unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q times dim^(-1/2). Returns
+        u [rows, channels + heads] 32-bit: q, k, v, and beta = sigmoid(proj[:, beta_off + head])."""
+        n = proj.shape[0]
+        C, K = taps.shape
+        if C != 2 * qk_heads * dim + n_heads * vdim:
+            raise KernelError(f"delta_prepare: {C} convolved channels for {qk_heads} x {dim} q and k and {n_heads} x {vdim} v")
+        self._f32_rows(proj, "delta_prepare projections", n, max(conv_off + C, beta_off + n_heads))
+        self._f32(taps, "conv taps", C * K)
+        self._check_lines("delta_prepare", state, conv_at + (K - 1) * C, batch)
+        self._index(batch.row_seq, "row_seq", n)
+        u = torch.empty(n, C + n_heads, dtype=torch.float32, device=self.device)
+        self._lazy("delta_rule").tis_delta_prepare(
+            _ptr(proj), proj.stride(0), int(conv_off), int(beta_off), _ptr(taps), K, _ptr(state), state.stride(0), int(conv_at),
+            _ptr(batch.row_seq), _ptr(batch.cu_rows), _ptr(batch.seq_slots), _ptr(u), u.stride(0), n, n_heads, qk_heads, dim,
+            vdim, self._stream())
+        return u
+
+    def delta_scan(self, u, q_off, k_off, v_off, beta_off, decay, state, batch, n_heads, qk_heads, dim, vdim):
+        """Walk the step's rows of every request through its matrix state, in order: per head S <- diag(decay) S;
+        w = beta (v - S^T k); S <- S + k w^T; o = S^T q. Returns o [rows, heads * vdim] 32-bit. u: [rows, ...] 32-bit with
+        q and k (qk_heads * dim each; head h reads those of qk head h // (heads / qk_heads)), v (heads * vdim) and beta
+        (heads) at the given columns; decay [rows, heads * dim]; state: [slots, floats] 32-bit, S [heads, dim, vdim] first."""
+        n = u.shape[0]
+        self._f32_rows(u, "delta_scan rows", n, max(q_off + qk_heads * dim, k_off + qk_heads * dim, v_off + n_heads * vdim,
+                                                    beta_off + n_heads))
+        self._f32_rows(decay, "delta_scan decays", n, n_heads * dim)
+        self._check_lines("delta_scan", state, n_heads * dim * vdim, batch)
+        out = torch.empty(n, n_heads * vdim, dtype=torch.float32, device=self.device)
+        self._lazy("delta_rule").tis_delta_scan(
+            _ptr(u), u.stride(0), int(q_off), int(k_off), int(v_off), int(beta_off), _ptr(decay), decay.stride(0), _ptr(state),
+            state.stride(0), _ptr(batch.cu_rows), _ptr(batch.seq_slots), batch.n_seqs, _ptr(out), out.stride(0), n_heads,
+            qk_heads, dim, vdim, self._stream())
         return out
 
     # ---- recurrent mixers with a matrix state per head ---------------------------------------------------
