@@ -216,9 +216,11 @@ def moe_ff(h, w, pre, mlp, margins=None):
         margins += mg
     limit = float(mlp["expert"]["limit"]) if E else 0.0
     y = torch.zeros_like(h)
-    for t in range(h.shape[0]):
-        for e, wt in zip(ids[t].tolist(), weights[t]):
-            y[t] += wt * (clamped_expert(h[t:t + 1], w, f"{pre}e{e}.", limit)[0] if e < E else h[t])
+    for e in range(E + I):
+        share = (weights * (ids == e)).sum(-1, keepdim=True)          # this output's weight per row, 0 where not chosen
+        rows = share[:, 0] != 0
+        if rows.any():
+            y[rows] += share[rows] * (clamped_expert(h[rows], w, f"{pre}e{e}.", limit) if e < E else h[rows])
     if mlp.get("shared"):
         shared = clamped_expert(h, w, pre + "shared.", float(mlp["shared"]["limit"]))
         y = y + shared * torch.sigmoid(h @ w[pre + "shared.sg"].t())
@@ -255,3 +257,12 @@ def forward(cfg, w, ids, layers_out=None, margins=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return rms_norm(x, w["final.norm"], eps) @ w["head"].t()
+
+
+def greedy_generate(cfg, w, prompt, n_new):
+    """The n_new tokens that follow `prompt` when the largest logit is taken every time (the whole sequence is run again
+    for every token: plain, not fast)."""
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(torch.argmax(forward(cfg, w, ids)[-1])))
+    return ids[len(prompt):]

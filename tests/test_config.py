@@ -40,7 +40,7 @@ def test_round_trip_through_a_folder(tmp_path):
     ({"D_MODEL": None}, "lacks 'D_MODEL'"),
     ({"NUM_GROUPS": None}, "lacks 'NUM_GROUPS'"),
     ({"architecture": None}, "lacks 'architecture'"),
-    ({"architecture": "Llama"}, "unknown architecture 'Llama'; known: Fikevik, Fipuzen, GqaMtpTransformer"),
+    ({"architecture": "Llama"}, "unknown architecture 'Llama'; known: Fesupel, Fikevik, Fipuzen, GqaMtpTransformer"),
     ({"N_HEAD": 7}, "not a multiple of n_heads"),
     ({"NUM_GROUPS": 5}, "not a multiple of the group size"),
     ({"D_MODEL": 36, "N_HEAD": 12}, "must be even"),
