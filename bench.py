@@ -18,7 +18,7 @@ with temperature, top-k, top-p and repetition penalty, finishing, pages given ba
     python bench.py --workload mixed --size 2.1B     64 requests decoding at contexts of 512..8192 while 2,048-token
                                                      portions of further prompts run in the same steps
 
-    python bench.py --workload designs               the Fikevik, Fipuzen and Rurorax designs beside the grouped-query decoder at equal
+    python bench.py --workload designs               the Fikevik, Fipuzen, Rurorax and Fesupel designs beside the grouped-query decoder at equal
                                                      sizes: prefill and decode throughput of each at a few layer sizes
 
 Each prints one line of the same form; `value` is generated tokens a second over the whole run (serve) or over the
@@ -338,6 +338,27 @@ def rurorax_config(width, heads, kv_heads, ff, layers, vocab, experts=8, top=2, 
                              "layers": [{"type": t, "mixer": m, "mlp": f} for t, m, f in (kinds[i % 4] for i in range(layers))]})
 
 
+def fesupel_config(width, heads, kv_heads, ff, layers, vocab, experts=8, top=2, chunk=1024):
+    """Every layer with attention of mixed sigmoid weights inside chunks beside a gated delta rule (heads / 2 heads of 128
+    key and 256 value channels: width channels in all, low-rank projections of 64); the feed-forward in turn dense
+    (ff wide) and a mixture of `experts` clamped gated experts and one identity expert in three groups of which two are
+    kept, a row taking `top`, each ff / top wide, beside a shared expert of ff / 4; a token input of 64 numbers a layer."""
+    from tiny_inference_server_amd.config import config_from_dict
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // top, "limit": 7.0},
+           "router": {"experts": experts, "identity": 1, "top": top, "groups": {"count": 3, "keep": 2}},
+           "shared": {"ff": ff // 4, "limit": 7.0}}
+    mixer = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+                      "mask": {"size": chunk},
+                      "rot": {"dims": 64, "base": 1000000.0, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+             "right": {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": 128, "vdim": 256, "conv": 4,
+                       "decay_rank": 64, "gate_rank": 64}}
+    return config_from_dict({"architecture": "Fesupel", "vocab": vocab, "width": width, "embedding": {"scale": width ** 0.5},
+                             "norm": {"eps": 1e-5}, "token_side": {"dim": 64},
+                             "layers": [{"type": "parallel", "mixer": mixer, "mlp": dense if i % 2 == 0 else moe}
+                                        for i in range(layers)]})
+
+
 def design_comparison(a, say):
     """Prefill (a.prefill_tokens tokens, one prompt) and decode (batch a.batch, context a.context) of the Fikevik and
     Fipuzen designs and of the grouped-query decoder without prediction heads at the sizes of DESIGN_SIZES, random
@@ -359,6 +380,7 @@ def design_comparison(a, say):
             "fikevik": fikevik_config(width, heads, kv_heads, ff, layers, vocab),
             "fipuzen": fipuzen_config(width, heads, kv_heads, ff, layers, vocab),
             "rurorax": rurorax_config(width, heads, kv_heads, ff, layers, vocab),
+            "fesupel": fesupel_config(width, heads, kv_heads, ff, layers, vocab),
             "gqa": GqaMtpConfig(d_model=width, vocab_size=vocab, max_context=max(8192, a.context), rope_base=500000.0,
                                 n_heads=heads, n_layers=layers, ffn_hidden=ff, group_size=heads // kv_heads, mtp_heads=0,
                                 rms_eps=1e-5, tie_embeddings=False),
@@ -417,7 +439,7 @@ def design_comparison(a, say):
             "warmup": a.warmup, "ms_per_step": points[first].get("decode_ms"), "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": dkey,
             "data": "synthetic: random weights N(0,0.02), uniform random token ids",
-            "config": {"model": "Fikevik, Fipuzen and Rurorax beside GqaMtpTransformer", "sizes": [list(s) for s in DESIGN_SIZES],
+            "config": {"model": "Fikevik, Fipuzen, Rurorax and Fesupel beside GqaMtpTransformer", "sizes": [list(s) for s in DESIGN_SIZES],
                        "global_batch": a.batch, "seq_len": a.context, "prefill_tokens": a.prefill_tokens,
                        "parallelism": "single-gpu"},
             "points": points}
@@ -445,7 +467,7 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", choices=["decode", "serve", "mixed", "designs"], default="decode")
     ap.add_argument("--requests", type=int, default=64, help="serve, mixed: requests (decoding at once)")
-    ap.add_argument("--designs", default="", help="designs: which of fikevik,fipuzen,rurorax,gqa to run (default: all)")
+    ap.add_argument("--designs", default="", help="designs: which of fikevik,fipuzen,rurorax,fesupel,gqa to run (default: all)")
     ap.add_argument("--design-sizes", default="", help="designs: which sizes to run, e.g. w2048 (default: all)")
     ap.add_argument("--phase", choices=["both", "prefill", "decode"], default="both", help="designs: what to measure")
     ap.add_argument("--new-tokens", type=int, default=256, help="serve: tokens generated per request")

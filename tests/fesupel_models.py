@@ -242,7 +242,7 @@ def sharpen(cfg, tensors, needle: int, probe: int, side: str = "left", strength:
     not mixed (rotation is left to the configuration: the tests' first layers rotate few channels slowly). side
     "right": q and k pass the convolution alone (the row's own tap is 1), the probe's q becomes the needle's k, the decay
     is made so slow that the state still holds the needle hundreds of tokens later, and beta is large at the needle
-    alone."""
+    alone (every token's embedding gets one channel in common, which the beta projection reads as a low bias)."""
     t = {n: v.float().clone() for n, v in tensors.items()}
     scale = float((cfg.get("embedding") or {}).get("scale", 1.0))
     eps = float(cfg["norm"]["eps"])
@@ -272,10 +272,18 @@ def sharpen(cfg, tensors, needle: int, probe: int, side: str = "left", strength:
         for n in ("q.conv", "k.conv"):
             t[p + n].zero_()
             t[p + n][:, -1] = 1.0
-        t[p + "q"] = looking(t[p + "k"]) * 4.0
+        # every token's first channel is the same large number, which the row of Wb below turns into a low beta for
+        # all tokens; the needle's own direction lifts its beta to about one
+        t["embed"][:, 0] = 3.0
+        hp, hn = normed(probe), normed(needle)
+        t[p + "q"] = (t[p + "k"] + torch.outer(t[p + "k"] @ (hn - hp), hp) / (hp @ hp)) * 4.0
         t[p + "k"] = t[p + "k"] * 4.0                      # silu of a larger number is nearer to the number itself
         t[p + "A_log"].fill_(-9.0)
-        t[p + "b"] = torch.outer(torch.full((m["heads"],), 8.0), hn - hp * (hn @ hp) / (hp @ hp)) / (hn @ hn)
+        first = torch.zeros_like(hn)
+        first[0] = 1.0
+        own = hn - first * hn[0]
+        own = own - (hp - first * hp[0]) * (own @ hp) / ((hp - first * hp[0]) @ hp)
+        t[p + "b"] = torch.outer(torch.ones(m["heads"]), -6.0 * first / hn[0] + 14.0 * own / (own @ hn))
     return {n: v.to(tensors[n].dtype) for n, v in t.items()}
 
 

@@ -376,3 +376,15 @@ def test_greedy_generation_through_the_scheduler():
         assert out == want
         assert s.peak_running == 2 and eng.cache.n_live == 0
         eng.cache.check()
+
+
+def test_the_named_size_runs_with_random_weights(tmp_path):
+    from tiny_inference_server_amd.__main__ import preset_names, size_config
+    from tiny_inference_server_amd.weights import write_random_model
+    assert "fesupel-small" in preset_names()
+    cfg = size_config("fesupel-small")
+    folder = write_random_model(cfg, 3, str(tmp_path / "m"))
+    assert load_config(folder).to_dict() == cfg.to_dict()
+    eng = Engine(folder, dtype="float32", max_tokens=64, max_requests=2, ops=TorchOps())
+    out = eng.step([("a", [5, 9, 1, 300], [3]), ("b", [7], [0])]).logits
+    assert out.shape == (2, cfg.vocab) and torch.isfinite(out).all()

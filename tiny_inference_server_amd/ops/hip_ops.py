@@ -1860,8 +1860,10 @@ class HipOps:
         partial = None
         if n_splits > 1:
             need = n * n_splits * n_heads * value_dim
-            partial = self._workspace if self._workspace.numel() >= need else torch.empty(need, dtype=torch.float32,
-                                                                                         device=self.device)
+            # (the fixed workspace where there is one and it is large enough; an allocation made while a graph is
+            # captured stays with the graph)
+            fits = self._workspace is not None and self._workspace.numel() >= need
+            partial = self._workspace if fits else torch.empty(need, dtype=torch.float32, device=self.device)
         self._lazy("attention_window").tis_attention_mixed(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), _ptr(partial), n_splits, n, n_heads, n_kv_heads, key_dim,

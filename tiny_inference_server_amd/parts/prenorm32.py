@@ -177,7 +177,7 @@ class SandwichStream32(PreNormStream32):
                 pad = -rows.shape[0] % 8
                 blocks.append(rows)
                 if pad:
-                    blocks.append(torch.zeros(pad, rows.shape[1], dtype=rows.dtype))
+                    blocks.append(torch.zeros(pad, rows.shape[1], dtype=rows.dtype, device=rows.device))
                 self.cols.append((at, at + rows.shape[0]))
                 at += rows.shape[0] + pad
             self.w_in = to_compute(ops, torch.cat(blocks, dim=0))

@@ -161,7 +161,7 @@ class PostNormGated(Arrangement):
             pad = -rows.shape[0] % 8
             blocks.append(rows)
             if pad:
-                blocks.append(torch.zeros(pad, rows.shape[1], dtype=rows.dtype))
+                blocks.append(torch.zeros(pad, rows.shape[1], dtype=rows.dtype, device=rows.device))
             at += rows.shape[0] + pad
             return first, first + rows.shape[0]
 
