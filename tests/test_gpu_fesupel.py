@@ -86,6 +86,38 @@ def test_attention_with_mixed_sigmoid_weights(dtype, Hq, G, kd, vd, chunk, cap):
         assert torch.isfinite(res[0].float()).all()
 
 
+@pytest.mark.parametrize("Hq,G,kd,vd,chunk,cap", [(4, 1, 64, 64, 100, 30.0), (16, 4, 128, 128, 333, 0.0), (5, 5, 24, 32, 7, 2.0), (6, 2, 40, 16, 0, 0.0),
+                                                  (2, 1, 128, 64, 64, 10.0), (13, 1, 16, 48, 1, 0.0), (8, 8, 32, 32, 1000, 5.0)])
+def test_matrix_core_attention_with_mixed_sigmoid_weights(Hq, G, kd, vd, chunk, cap):
+    """bfloat16 and pages of 16 slots: tiles of rows that cross chunk edges and page borders, a portion that goes on in the
+    middle of a page beside a new request, and single rows whose keys are cut over many workgroups; the pool is full of
+    NaN where nothing was written."""
+    ops, ref = hip_ops("bfloat16"), TorchOps("cpu", torch.bfloat16)
+    g = torch.Generator().manual_seed(kd + chunk)
+    ps, n_pages = 16, 40
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    tables = [perm[:18] + [0, 0], perm[18:38]]
+    cols = Hq * kd + G * kd + G * vd
+    head_bias, talk = torch.randn(Hq, generator=g) - 2, torch.eye(Hq) + 0.4 * torch.randn(Hq, Hq, generator=g)
+    planes = [torch.full((n_pages, G * ps * (kd + vd)), float("nan"), dtype=torch.bfloat16) for _ in range(2)]
+    planes[0] = planes[0].cuda()
+    for seq_rows, slots, tabs in (([(0, 0, 203)], [0], [tables[1]]), ([(0, 0, 37), (37, 203, 70)], [1, 0], [tables[0], tables[1]]),
+                                  ([(0, 37, 1), (1, 273, 1)], [1, 0], [tables[0], tables[1]]),
+                                  ([(0, 38, 2), (2, 274, 1), (3, 0, 0)][:2], [1, 0], [tables[0], tables[1]])):
+        n = sum(r[2] for r in seq_rows)
+        proj = torch.randn(n, cols, generator=g)
+        res = []
+        for o, plane, dev in ((ops, planes[0], "cuda"), (ref, planes[1], "cpu")):
+            b = fake_batch(seq_rows, slots, tabs, ps, dev)
+            q = o.attention_prepare(proj.to(dev), 0, Hq * kd, Hq * kd + G * kd, b.positions, b.write_slots["g"], plane, Hq, G, kd, vd,
+                                    ps, value_norm=False)
+            res.append(o.mixed_sigmoid_attention(q, plane, b, "g", Hq, G, kd, vd, ps, chunk, kd ** -0.5, cap, head_bias.to(dev),
+                                                 talk.to(dev)))
+        assert ops._mixed_on_matrix_cores(res[0], kd, vd, ps, Hq)
+        assert torch.isfinite(res[0].float()).all()
+        close(res[0], res[1], "bfloat16", f"attention of {seq_rows}", tol=2.5e-2)
+
+
 def test_attention_of_many_rows_and_long_chunks():
     """Hundreds of rows (one workgroup a row, no key splits) over chunks longer than a block of keys."""
     ops, ref = hip_ops("float32"), TorchOps("cpu", torch.float32)

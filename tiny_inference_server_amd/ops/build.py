@@ -47,6 +47,7 @@ SOURCES: Dict[str, str] = {
     "attention_latent": "attention_latent.hip",
     "ssm_parts": "ssm_parts.hip",
     "delta_rule": "delta_rule.hip",
+    "attention_mixed": "attention_mixed.hip",
 }
 HEADERS = ["common.h", "attention_mfma.h"]
 # what a library links beyond the HIP runtime
@@ -85,6 +86,8 @@ VARIANTS: Dict[str, tuple] = {
     "attention_mfma": ("TIS_HD", (32, 48, 64, 128, 256)),
     # keys' channels * 10000 + values' channels of a latent (others are built when a model first asks for them)
     "attention_latent": ("TIS_LATENT", (5760512,)),
+    # keys' channels * 100000 + values' channels * 100 + heads a wave takes (others are built when a model first asks)
+    "attention_mixed": ("TIS_AMX", (12812804, 6406401)),
 }
 
 

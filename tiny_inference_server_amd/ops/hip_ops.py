@@ -155,6 +155,10 @@ _SIGNATURES["delta_rule"] = ("tis_delta_rule", {
     "tis_delta_scan": [_P, _L, _I, _I, _I, _I, _P, _L, _P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _I, _P],
 })
 
+_SIGNATURES["attention_mixed"] = ("tis_attention_mixed", {
+    "tis_attention_mixed_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _P, _L, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P, _P, _P],
+})
+
 _libs = {}
 
 
@@ -1824,6 +1828,19 @@ class HipOps:
             gate.stride(0) if gate is not None else 0, self._stream())
         return out
 
+    def plan_row_tiles(self, seq_rows, add):
+        """Host planning for the matrix-core attention with mixed sigmoid weights: its items for a step's rows, (first
+        row, rows) each, up to 16 consecutive rows of one request. Steps of single rows need no list."""
+        if self.dtype != torch.bfloat16 or all(n <= 1 for _, _, n in seq_rows):
+            return {}
+        items = latent_items(seq_rows, 1, 16)
+        return {("row_tiles", 16): (add(items), len(items))}
+
+    def _mixed_on_matrix_cores(self, q, key_dim, value_dim, page_size, n_heads):
+        return (self.dtype == torch.bfloat16 and page_size == 16 and key_dim % 8 == 0 and value_dim % 16 == 0
+                and key_dim <= 512 and value_dim <= 512 and n_heads <= 28 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0
+                and -(-n_heads // 4) * (value_dim // 16 + key_dim // 32) <= 64)
+
     def mixed_sigmoid_attention(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, chunk,
                                 scale, softcap, head_bias, talk):
         """Attention of the rows in `batch` whose weights are sigmoids mixed across the heads: for every key j that the
@@ -1849,13 +1866,36 @@ class HipOps:
         out = self.empty(n, n_heads * value_dim)
         if n == 0:
             return out
+        longest = min(batch.max_kv_len, chunk) if chunk > 0 else batch.max_kv_len
+        if self._mixed_on_matrix_cores(q, key_dim, value_dim, page_size, n_heads):
+            # bfloat16 with pages of 16 slots: four waves an item of up to 16 rows, a library per sizes (compiled when a
+            # model first asks for it)
+            items, n_items = None, n
+            if batch.max_seq_rows > 1:
+                plan = batch.extras.get(("row_tiles", 16))
+                if plan is None:        # a caller that did not plan (a kernel test)
+                    host = latent_items(batch.seq_rows, 1, 16)
+                    plan = (torch.from_numpy(host).reshape(-1).to(self.device), len(host))
+                items, n_items = plan[0].reshape(-1), plan[1]
+                if items.numel() < 2 * n_items or items.dtype != torch.int32 or not items.is_contiguous():
+                    raise KernelError(f"attention: a list of {items.numel()} integers for {n_items} items")
+            # few items: an item's keys are cut over several workgroups (two a compute unit), whose parts are added up
+            most = max(1, self._workspace.numel() // (n * n_heads * value_dim))
+            n_splits = int(max(1, min(-(-(longest + 31) // 32), (2 * self.units) // n_items, 64, most)))
+            hpw = -(-n_heads // 4)
+            lib = self._lazy(f"attention_mixed@{key_dim * 100000 + value_dim * 100 + hpw}")
+            lib.tis_attention_mixed_mfma(
+                _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq), _ptr(batch.positions),
+                _ptr(items), n_items, _ptr(out), out.stride(0), _ptr(self._workspace if n_splits > 1 else None), n_splits, n,
+                n_heads, n_kv_heads, key_dim, value_dim, page_size, int(chunk), float(scale), float(softcap), _ptr(head_bias),
+                _ptr(talk), self._stream())
+            return out
         # keys a workgroup takes at a time: what LDS holds beside the row's queries, in whole pages
         room = (16384 - n_heads * key_dim - n_heads * n_heads) // (2 * n_heads)
         block = min(256, room // 16 * 16 if room >= 16 else room)
         if block < 1:
             raise KernelError(f"attention: {n_heads} heads of {key_dim} channels do not fit the kernel for any sizes")
         # few rows: a row's keys are cut over several workgroups, whose parts a second kernel adds up
-        longest = min(batch.max_kv_len, chunk) if chunk > 0 else batch.max_kv_len
         n_splits = int(max(1, min(-(-longest // block), (2 * self.units) // n, 64)))
         partial = None
         if n_splits > 1:

@@ -509,6 +509,13 @@ class SigmoidMixedAttention:
         self.talk = to_gain(ops, tensors.of(spec, "talk"))
         self.w_o = to_compute(ops, tensors.of(spec, "o"))
 
+    # the matrix-core kernel's items (tiles of up to 16 rows of one request), where a step brings portions
+    def plan_key(self):
+        return ("row_tiles", 16) if hasattr(self.ops, "plan_row_tiles") else None
+
+    def plan_rows(self, seq_rows, add, mode=None):
+        return self.ops.plan_row_tiles(seq_rows, add)
+
     def core(self, proj, ctx):
         ops, b = self.ops, ctx.batch
         q = ops.attention_prepare(proj, 0, self.k_at, self.v_at, b.positions, b.write_slots[ctx.group], ctx.plane, self.H,
