@@ -78,82 +78,150 @@ __global__ __launch_bounds__(TIS_WAVE) void delta_prepare_kernel(
   for (int h = lane; h < H; h += TIS_WAVE) out[r * ldo + C + h] = dr_sigmoid(proj[r * ldp + beta_off + h]);
 }
 
-// The walk. grid (requests, heads, blocks of 16 value channels), 256 threads: thread (c, l) = (t / 16, t % 16) owns, for
+// Sum over the 16 lanes of a row of lanes (lanes 16 r .. 16 r + 15), every lane gets it: four data-parallel moves
+// inside the row (two inside quads, then the half row and the row mirrored), no trip through LDS. One fixed order.
+__device__ __forceinline__ float dr_row_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));   // row_mirror
+  return v;
+}
+
+// The walk. grid (blocks of 16 value channels, heads, requests), 256 threads: thread (c, l) = (t / 16, t % 16) owns, for
 // value channel c, the state's key channels [l * R, (l + 1) * R) in registers from the line before the first row to the
-// line after the last. A token's two sums over the key channels (S^T k and S^T q) are R terms a lane and a butterfly over
-// the 16 lanes of a column: every state element sees its rows strictly in order and every sum has one fixed order, so a
-// row's result does not depend on how its prompt was cut or on what else is in the step, bit for bit. Rows come through
-// LDS `tokens` at a time: [tokens][k: D | decay: D | q: D | v: 16 | beta: 1].
+// line after the last (the line goes through LDS both ways, so that memory sees whole runs of 16 channels). With
+// S' = diag(a) S, a token needs S'^T k for its write and (S' + k w^T)^T q = S'^T q + (k . q) w for its read: the three
+// sums over the key channels (S'^T k, S'^T q, k . q) are R terms a lane each and then one pass over the 16 lanes of a
+// column for all three together. Every state element sees its rows strictly in order and every sum has one fixed
+// order, so a row's result does not depend on how its prompt was cut or on what else is in the step, bit for bit.
+// Rows come through LDS 16 at a time (8 where a lane holds 16 key channels): [rows][k: Dp | decay: Dp | q: Dp | v: 16 | beta | 3 unused].
 template <int R>
 __global__ __launch_bounds__(256) void delta_scan_kernel(
     const float* __restrict__ u, long ldu, int q_off, int k_off, int v_off, int beta_off, const float* __restrict__ decay,
     long ldd, float* __restrict__ state, long lds, const int* __restrict__ cu_rows, const int* __restrict__ seq_slots,
     float* __restrict__ out, long ldo, int H, int G, int D, int V, int tokens) {
-  extern __shared__ float dr_lds[];
-  const int s = blockIdx.x, h = blockIdx.y, vb = blockIdx.z, t = threadIdx.x;
+  extern __shared__ __attribute__((aligned(16))) float dr_lds[];
+  const int s = blockIdx.z, h = blockIdx.y, vb = blockIdx.x, t = threadIdx.x;
   const int first = cu_rows[s], n_rows = cu_rows[s + 1] - first;
   if (n_rows <= 0) return;
-  const int c = vb * 16 + t / 16, l = t % 16;
+  const int cl = t / 16, l = t % 16;
+  const int c = vb * 16 + cl;
   const bool live = c < V;
   const int hq = h / (H / G);
-  const int Dp = 16 * R;                     // key channels as the lanes hold them (those from D on are zeros)
-  const int stride = 3 * Dp + 17;
+  constexpr int Dp = 16 * R;                 // key channels as the lanes hold them (those from D on are zeros)
+  constexpr int stride = 3 * Dp + 20;
   float* S_line = state + (long)seq_slots[s] * lds + (long)h * D * V;
+  // the line's [D][16 channels of this block] into LDS in runs of 16, then each lane's own elements
+  for (int e = t; e < D * 16; e += 256) {
+    const int d = e / 16, cc = vb * 16 + e % 16;
+    dr_lds[e] = cc < V ? S_line[(long)d * V + cc] : 0.f;
+  }
+  __syncthreads();
   float S[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int d = l * R + i;
-    S[i] = (live && d < D) ? S_line[(long)d * V + c] : 0.f;
+    S[i] = d < D ? dr_lds[d * 16 + cl] : 0.f;
   }
-  for (int r0 = 0; r0 < n_rows; r0 += tokens) {
-    const int n = min(tokens, n_rows - r0);
-    __syncthreads();
-    for (int i = t; i < n * Dp; i += 256) {
-      const int tt = i / Dp, d = i % Dp;
+  // Rows go through two LDS buffers: while one chunk of rows is walked, the next one's loads are in flight in registers
+  // and are put into the other buffer afterwards, so one barrier a chunk and no wait for memory between chunks.
+  constexpr int TOK = R <= 8 ? 16 : 8;       // rows a chunk (`tokens`)
+  constexpr int NI = TOK * Dp / 256;         // k, decay and q elements a thread fetches for a chunk
+  float pk[NI], pa[NI], pq[NI], pv[2];
+  auto fetch = [&](int r0) {
+    const int n = min(TOK, n_rows - r0);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int i = t + 256 * j, tt = i / Dp, d = i % Dp;
       const long row = first + r0 + tt;
-      float* dst = dr_lds + tt * stride;
-      dst[d] = d < D ? u[row * ldu + k_off + hq * D + d] : 0.f;
-      dst[Dp + d] = d < D ? decay[row * ldd + h * D + d] : 0.f;
-      dst[2 * Dp + d] = d < D ? u[row * ldu + q_off + hq * D + d] : 0.f;
+      const bool ok = tt < n && d < D;
+      pk[j] = ok ? u[row * ldu + k_off + hq * D + d] : 0.f;
+      pa[j] = ok ? decay[row * ldd + h * D + d] : 0.f;
+      pq[j] = ok ? u[row * ldu + q_off + hq * D + d] : 0.f;
     }
-    for (int i = t; i < n * 17; i += 256) {
-      const int tt = i / 17, j = i % 17;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int i = t + 256 * j, tt = i / 17, e = i % 17;
       const long row = first + r0 + tt;
-      const int cc = vb * 16 + j;
-      dr_lds[tt * stride + 3 * Dp + j] = j == 16 ? u[row * ldu + beta_off + h] : (cc < V ? u[row * ldu + v_off + h * V + cc] : 0.f);
+      const int cc = vb * 16 + e;
+      pv[j] = tt < n ? (e == 16 ? u[row * ldu + beta_off + h] : (cc < V ? u[row * ldu + v_off + h * V + cc] : 0.f)) : 0.f;
     }
-    __syncthreads();
+  };
+  auto commit = [&](float* buf) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int i = t + 256 * j, tt = i / Dp, d = i % Dp;
+      float* dst = buf + tt * stride;
+      dst[d] = pk[j];
+      dst[Dp + d] = pa[j];
+      dst[2 * Dp + d] = pq[j];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int i = t + 256 * j, tt = i / 17, e = i % 17;
+      if (tt < TOK) buf[tt * stride + 3 * Dp + e] = pv[j];
+    }
+  };
+  __syncthreads();               // every lane has taken its part of the line out of LDS
+  fetch(0);
+  commit(dr_lds);
+  __syncthreads();
+  int which = 0;
+  for (int r0 = 0; r0 < n_rows; r0 += TOK, which ^= 1) {
+    const int n = min(TOK, n_rows - r0);
+    const bool more = r0 + TOK < n_rows;
+    if (more) fetch(r0 + TOK);
+    const float* rows_lds = dr_lds + which * (TOK * stride);
     for (int tt = 0; tt < n; ++tt) {
-      const float* src = dr_lds + tt * stride;
-      const float* kk = src + l * R;
-      const float* aa = src + Dp + l * R;
-      const float* qq = src + 2 * Dp + l * R;
-      float kv[R];
-      float dot = 0.f;
+      const float* src = rows_lds + tt * stride;
+      float kv[R], av[R], qv[R];
+      if constexpr (R % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < R; i += 4) {
+          const float4 a = *reinterpret_cast<const float4*>(src + l * R + i);
+          const float4 b = *reinterpret_cast<const float4*>(src + Dp + l * R + i);
+          const float4 q4 = *reinterpret_cast<const float4*>(src + 2 * Dp + l * R + i);
+          kv[i] = a.x, kv[i + 1] = a.y, kv[i + 2] = a.z, kv[i + 3] = a.w;
+          av[i] = b.x, av[i + 1] = b.y, av[i + 2] = b.z, av[i + 3] = b.w;
+          qv[i] = q4.x, qv[i + 1] = q4.y, qv[i + 2] = q4.z, qv[i + 3] = q4.w;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+          kv[i] = src[l * R + i];
+          av[i] = src[Dp + l * R + i];
+          qv[i] = src[2 * Dp + l * R + i];
+        }
+      }
+      float dk = 0.f, dq = 0.f, kq = 0.f;
 #pragma unroll
       for (int i = 0; i < R; ++i) {
-        kv[i] = kk[i];
-        S[i] *= aa[i];
-        dot += S[i] * kv[i];
+        S[i] *= av[i];
+        dk += S[i] * kv[i];
+        dq += S[i] * qv[i];
+        kq += kv[i] * qv[i];
       }
+      dk = dr_row_sum(dk);
+      dq = dr_row_sum(dq);
+      kq = dr_row_sum(kq);
+      const float w = src[3 * Dp + 16] * (src[3 * Dp + cl] - dk);
 #pragma unroll
-      for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, TIS_WAVE);
-      const float w = src[3 * Dp + 16] * (src[3 * Dp + t / 16] - dot);
-      float res = 0.f;
-#pragma unroll
-      for (int i = 0; i < R; ++i) {
-        S[i] += kv[i] * w;
-        res += S[i] * qq[i];
-      }
-#pragma unroll
-      for (int o = 8; o > 0; o >>= 1) res += __shfl_xor(res, o, TIS_WAVE);
-      if (live && l == 0) out[(long)(first + r0 + tt) * ldo + h * V + c] = res;
+      for (int i = 0; i < R; ++i) S[i] += kv[i] * w;
+      if (live && l == 0) out[(long)(first + r0 + tt) * ldo + h * V + c] = dq + kq * w;
     }
+    if (more) commit(dr_lds + (which ^ 1) * (TOK * stride));
+    __syncthreads();
   }
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int d = l * R + i;
-    if (live && d < D) S_line[(long)d * V + c] = S[i];
+    if (d < D) dr_lds[d * 16 + cl] = S[i];
+  }
+  __syncthreads();
+  for (int e = t; e < D * 16; e += 256) {
+    const int d = e / 16, cc = vb * 16 + e % 16;
+    if (cc < V) S_line[(long)d * V + cc] = dr_lds[e];
   }
 }
 
@@ -176,12 +244,13 @@ TIS_EXPORT int tis_delta_scan(const float* u, long ldu, int q_off, int k_off, in
                               long ldd, float* state, long lds, const int* cu_rows, const int* seq_slots, int n_seqs,
                               float* out, long ldo, int H, int G, int D, int V, hipStream_t stream) {
   if (n_seqs == 0) return 0;
-  if (n_seqs < 0 || H < 1 || H > 65535 || G < 1 || H % G || D < 1 || D > 256 || V < 1 || (V + 15) / 16 > 65535)
+  if (n_seqs < 0 || n_seqs > 65535 || H < 1 || H > 65535 || G < 1 || H % G || D < 1 || D > 256 || V < 1)
     return tis_fail("delta_scan: bad size requests=%d heads=%d qk_heads=%d dim=%d (at most 256) vdim=%d", n_seqs, H, G, D, V);
   const int R = D <= 16 ? 1 : D <= 32 ? 2 : D <= 64 ? 4 : D <= 128 ? 8 : 16;
   const int tokens = R <= 8 ? 16 : 8;
-  const size_t lds_bytes = (size_t)tokens * (3 * 16 * R + 17) * sizeof(float);
-  dim3 grid(n_seqs, H, (V + 15) / 16);
+  size_t lds_bytes = 2 * (size_t)tokens * (3 * 16 * R + 20) * sizeof(float);      // two buffers of rows
+  if (lds_bytes < (size_t)D * 16 * sizeof(float)) lds_bytes = (size_t)D * 16 * sizeof(float);      // the line's way in and out
+  dim3 grid((V + 15) / 16, H, n_seqs);
 #define DR_SCAN(RR)                                                                                                        \
   delta_scan_kernel<RR><<<grid, 256, lds_bytes, stream>>>(u, ldu, q_off, k_off, v_off, beta_off, decay, ldd, state, lds,   \
                                                           cu_rows, seq_slots, out, ldo, H, G, D, V, tokens)
