@@ -102,24 +102,34 @@ __global__ __launch_bounds__(256) void attention_mixed_mfma_kernel(
       page_ok[t] = key0 <= p_hi;
       base[t] = plane + (long)bt[(page_ok[t] ? key0 : p_hi) / PAGE] * page_stride;
     }
-    // scores and weights of this wave's heads
+    // scores and weights of this wave's heads; the keys of a key/value head are fetched once for the heads that share it
+    bf16x8 ka[2][DC];
+    int kv_have = -1;
 #pragma unroll
     for (int u = 0; u < HPW; ++u) {
       const int h = wave * HPW + u;
       if (h < H) {
-        const long k_head = (long)(h / group_size) * PAGE * KD;
+        const int kv_head = h / group_size;
+        if (kv_head != kv_have) {
+          kv_have = kv_head;
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const bf16* kp = base[t] + (long)kv_head * PAGE * KD + (long)c16 * KD;
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) {
+              const int d = dc * 32 + g4 * 8;
+              const bool ok = d < KD;
+              const bf16x8 kv = amx_load8(kp + (ok ? d : 0));
+              ka[t][dc] = ok ? kv : (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+            }
+          }
+        }
         f32x4 st[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
           st[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-          const bf16* kp = base[t] + k_head + (long)c16 * KD;
 #pragma unroll
-          for (int dc = 0; dc < DC; ++dc) {
-            const int d = dc * 32 + g4 * 8;
-            const bool ok = d < KD;
-            const bf16x8 kv = amx_load8(kp + (ok ? d : 0));
-            st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ok ? kv : (bf16x8){0, 0, 0, 0, 0, 0, 0, 0}, qb[u][dc], st[t], 0, 0, 0);
-          }
+          for (int dc = 0; dc < DC; ++dc) st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[t][dc], qb[u][dc], st[t], 0, 0, 0);
         }
         float w[8];
 #pragma unroll
@@ -128,7 +138,8 @@ __global__ __launch_bounds__(256) void attention_mixed_mfma_kernel(
           for (int i = 0; i < 4; ++i) {
             const int j = s * 32 + t * 16 + g4 * 4 + i;
             float x = st[t][i] * scale;
-            if (softcap > 0.f) x = softcap * tanhf(x * inv_cap);
+            // tanh(y) = 1 - 2 / (1 + exp(2 y)), on the fast exponential (|y| is capped so that exp stays finite)
+            if (softcap > 0.f) x = softcap * (1.f - 2.f / (1.f + __expf(2.f * fminf(fmaxf(x * inv_cap, -15.f), 15.f))));
             const float sg = 1.f / (1.f + __expf(-(x + hb[u])));
             w[t * 4 + i] = (row_ok && j <= p_row && j >= lo_row) ? sg : 0.f;
           }

@@ -599,24 +599,40 @@ TIS_EXPORT int tis_softcap(float* z, long ldz, float cap, int rows, int W, hipSt
 // out[r][c] = act(z) with z = sum_k low[r][k] * w2[c][k] + bias[c] (bias may be null): the second half of a low-rank
 // projection, in 32-bit. kind 0: sigmoid(z)^(1/tau); 1: exp(-rate[c / group] * softplus(z)), a decay whose rate is one
 // number per run of `group` channels; 2: z itself.
+static constexpr int LR_ROWS = 8;      // rows a workgroup of lowrank_act takes: a channel's line of w2 is read once for them
+
 __global__ __launch_bounds__(S32_THREADS) void lowrank_act_kernel(const float* __restrict__ low, long ldl, int rank,
                                                                    const float* __restrict__ w2,
                                                                    const float* __restrict__ bias, int kind, float tau,
                                                                    const float* __restrict__ rate, int group,
-                                                                   float* __restrict__ out, int C, int row_blocks) {
-  extern __shared__ float a[];
-  const long r = blockIdx.x / row_blocks;        // a row's blocks of channels side by side: a few rows still fill the chip
-  for (int k = threadIdx.x; k < rank; k += S32_THREADS) a[k] = low[r * ldl + k];
+                                                                   float* __restrict__ out, int rows, int C, int col_blocks) {
+  extern __shared__ float a[];                   // [LR_ROWS][rank]
+  // grid (blocks of rows * blocks of channels, a row block's side by side): a few rows still fill the chip
+  const long r0 = (long)(blockIdx.x / col_blocks) * LR_ROWS;
+  const int n = (int)min((long)LR_ROWS, rows - r0);
+  for (int i = threadIdx.x; i < n * rank; i += S32_THREADS) a[i] = low[(r0 + i / rank) * ldl + i % rank];
   __syncthreads();
-  const int c = (blockIdx.x % row_blocks) * S32_THREADS + threadIdx.x;
+  const int c = (blockIdx.x % col_blocks) * S32_THREADS + threadIdx.x;
   if (c >= C) return;
-  float z = 0.f;
+  float z[LR_ROWS];
+#pragma unroll
+  for (int r = 0; r < LR_ROWS; ++r) z[r] = 0.f;
   const float* w = w2 + (long)c * rank;
-  for (int k = 0; k < rank; ++k) z += a[k] * w[k];
-  if (bias) z += bias[c];
-  if (kind == 0) z = expf(log_sigmoid_f(z) / tau);
-  else if (kind == 1) z = expf(-rate[c / group] * (z > 20.f ? z : log1pf(expf(z))));
-  out[r * C + c] = z;
+  for (int k = 0; k < rank; ++k) {
+    const float wk = w[k];
+#pragma unroll
+    for (int r = 0; r < LR_ROWS; ++r) z[r] += a[(r < n ? r : 0) * rank + k] * wk;      // (k in rising order for every row)
+  }
+  const float b = bias ? bias[c] : 0.f;
+  const float rt = kind == 1 ? rate[c / group] : 0.f;
+#pragma unroll
+  for (int r = 0; r < LR_ROWS; ++r) {
+    if (r >= n) break;
+    float v = z[r] + b;
+    if (kind == 0) v = expf(log_sigmoid_f(v) / tau);
+    else if (kind == 1) v = expf(-rt * (v > 20.f ? v : log1pf(expf(v))));
+    out[(r0 + r) * C + c] = v;
+  }
 }
 
 // out[r] = (1 / n) * sum_i y_i[r] / sqrt(mean(y_i[r]^2) + eps) * gain_i: the mean of one or two RMS-normed rows, 32-bit.
@@ -667,9 +683,11 @@ TIS_EXPORT int tis_lowrank_act(const float* low, long ldl, int rank, const float
   if (rows < 0 || rank < 1 || rank > 8192 || C < 1 || kind < 0 || kind > 2 || (kind == 0 && !(tau > 0.f)) ||
       (kind == 1 && (!rate || group < 1)))
     return tis_fail("lowrank_act: bad arguments rows=%d rank=%d channels=%d kind=%d", rows, rank, C, kind);
-  const int row_blocks = (C + S32_THREADS - 1) / S32_THREADS;
-  lowrank_act_kernel<<<(long)rows * row_blocks, S32_THREADS, rank * sizeof(float), stream>>>(low, ldl, rank, w2, bias, kind, tau,
-                                                                                            rate, group, out, C, row_blocks);
+  const int col_blocks = (C + S32_THREADS - 1) / S32_THREADS;
+  const long row_blocks = ((long)rows + LR_ROWS - 1) / LR_ROWS;
+  if (rank > 1024) return tis_fail("lowrank_act: rank %d (at most 1024)", rank);
+  lowrank_act_kernel<<<row_blocks * col_blocks, S32_THREADS, LR_ROWS * rank * sizeof(float), stream>>>(
+      low, ldl, rank, w2, bias, kind, tau, rate, group, out, rows, C, col_blocks);
   return tis_launch_status("lowrank_act");
 }
 
