@@ -173,36 +173,27 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     const bool more = r0 + TOK < n_rows;
     if (more) fetch(r0 + TOK);
     const float* rows_lds = dr_lds + which * (TOK * stride);
-    // a token's k, decay and q are read from LDS while the token before it is computed
-    float kv[R], av[R], qv[R], kn[R], an[R], qn[R];
-    auto read = [&](int tt, float (&k_)[R], float (&a_)[R], float (&q_)[R]) {
+    for (int tt = 0; tt < n; ++tt) {
       const float* src = rows_lds + tt * stride;
+      float kv[R], av[R], qv[R];
       if constexpr (R % 4 == 0) {
 #pragma unroll
         for (int i = 0; i < R; i += 4) {
           const float4 a = *reinterpret_cast<const float4*>(src + l * R + i);
           const float4 b = *reinterpret_cast<const float4*>(src + Dp + l * R + i);
           const float4 q4 = *reinterpret_cast<const float4*>(src + 2 * Dp + l * R + i);
-          k_[i] = a.x, k_[i + 1] = a.y, k_[i + 2] = a.z, k_[i + 3] = a.w;
-          a_[i] = b.x, a_[i + 1] = b.y, a_[i + 2] = b.z, a_[i + 3] = b.w;
-          q_[i] = q4.x, q_[i + 1] = q4.y, q_[i + 2] = q4.z, q_[i + 3] = q4.w;
+          kv[i] = a.x, kv[i + 1] = a.y, kv[i + 2] = a.z, kv[i + 3] = a.w;
+          av[i] = b.x, av[i + 1] = b.y, av[i + 2] = b.z, av[i + 3] = b.w;
+          qv[i] = q4.x, qv[i + 1] = q4.y, qv[i + 2] = q4.z, qv[i + 3] = q4.w;
         }
       } else {
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-          k_[i] = src[l * R + i];
-          a_[i] = src[Dp + l * R + i];
-          q_[i] = src[2 * Dp + l * R + i];
+          kv[i] = src[l * R + i];
+          av[i] = src[Dp + l * R + i];
+          qv[i] = src[2 * Dp + l * R + i];
         }
       }
-    };
-    read(0, kn, an, qn);
-    for (int tt = 0; tt < n; ++tt) {
-      const float* src = rows_lds + tt * stride;
-      const float beta = src[3 * Dp + 16], val = src[3 * Dp + cl];
-#pragma unroll
-      for (int i = 0; i < R; ++i) kv[i] = kn[i], av[i] = an[i], qv[i] = qn[i];
-      if (tt + 1 < n) read(tt + 1, kn, an, qn);
       float dk = 0.f, dq = 0.f, kq = 0.f;
 #pragma unroll
       for (int i = 0; i < R; ++i) {
@@ -214,7 +205,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
       dk = dr_row_sum(dk);
       dq = dr_row_sum(dq);
       kq = dr_row_sum(kq);
-      const float w = beta * (val - dk);
+      const float w = src[3 * Dp + 16] * (src[3 * Dp + cl] - dk);
 #pragma unroll
       for (int i = 0; i < R; ++i) S[i] += kv[i] * w;
       if (live && l == 0) out[(long)(first + r0 + tt) * ldo + h * V + c] = dq + kq * w;
