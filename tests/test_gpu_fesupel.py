@@ -146,8 +146,10 @@ def test_the_delta_rules_kernels(Hh, G, D, V, K):
     C = 2 * G * D + Hh * V
     cols = 5 + C + Hh
     taps = torch.randn(C, K, generator=g) / K ** 0.5
-    floats = Hh * D * V + (K - 1) * C
-    states = [torch.zeros(3, floats + 3), torch.zeros(3, floats + 3).cuda()]
+    at = Hh * -(-V // 16) * D * 16           # the matrix state in blocks of 16 value channels, then the convolution's inputs
+    floats = at + (K - 1) * C
+    floats += -floats % 4 + 4                # lines start 16 bytes aligned
+    states = [torch.zeros(3, floats), torch.zeros(3, floats).cuda()]
     for seq_rows, slots in (([(0, 0, 37)], [2]), ([(0, 37, 1), (1, 0, 9)], [2, 0]), ([(0, 9, 70), (70, 38, 2)], [0, 2]),
                             ([(0, 40, 1), (1, 79, 1)], [2, 0])):
         n = sum(r[2] for r in seq_rows)
@@ -156,8 +158,8 @@ def test_the_delta_rules_kernels(Hh, G, D, V, K):
         res = []
         for o, st, dev in ((ref, states[0], "cpu"), (ops, states[1], "cuda")):
             b = fake_batch(seq_rows, slots, None, 8, dev)
-            u = o.delta_prepare(proj.to(dev), 5, 5 + C, taps.to(dev), st, Hh * D * V, b, Hh, G, D, V)
-            o.conv_state_update(proj.to(dev), 5, C, K, st, Hh * D * V, b)
+            u = o.delta_prepare(proj.to(dev), 5, 5 + C, taps.to(dev), st, at, b, Hh, G, D, V)
+            o.conv_state_update(proj.to(dev), 5, C, K, st, at, b)
             res.append((u, o.delta_scan(u, 0, G * D, 2 * G * D, C, decay.to(dev), st, b, Hh, G, D, V)))
         close(res[1][0], res[0][0], "float32", "prepared rows", tol=1e-5)
         close(res[1][1], res[0][1], "float32", "outputs", tol=1e-4)

@@ -495,8 +495,13 @@ class TorchOps:
         out = torch.zeros(n, H * V, dtype=torch.float32)
         cu, slots = batch.cu_rows.tolist(), batch.seq_slots.tolist()
         rep = H // G
+        VB = -(-V // 16)
         for s in range(batch.n_seqs):
-            S = state[slots[s], :H * D * V].view(H, D, V)
+            if cu[s + 1] == cu[s]:
+                continue
+            # the line holds S as [heads, blocks of 16 value channels, dim, 16]
+            line = state[slots[s], :H * VB * D * 16].view(H, VB, D, 16)
+            S = line.permute(0, 2, 1, 3).reshape(H, D, VB * 16)[:, :, :V].clone()
             for r in range(cu[s], cu[s + 1]):
                 q = u[r, q_off:q_off + G * D].view(G, D).repeat_interleave(rep, dim=0)
                 k = u[r, k_off:k_off + G * D].view(G, D).repeat_interleave(rep, dim=0)
@@ -506,6 +511,9 @@ class TorchOps:
                 w = beta[:, None] * (v - torch.einsum("hdv,hd->hv", S, k))
                 S.add_(k[:, :, None] * w[:, None, :])
                 out[r] = torch.einsum("hdv,hd->hv", S, q).reshape(-1)
+            full = torch.zeros(H, D, VB * 16)
+            full[:, :, :V] = S
+            line.copy_(full.view(H, D, VB, 16).permute(0, 2, 1, 3))
         return out
 
     # ---- attention whose weights are sigmoids mixed across the heads --------------------------------------------

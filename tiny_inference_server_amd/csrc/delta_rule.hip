@@ -2,11 +2,13 @@
 //
 //   S <- diag(a_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
 //
-// per head and row, S being [key channels][value channels] 32-bit floats in the request's state line. Two kernels: the
+// per head and row, S being 32-bit floats in the request's state line, laid out [head][block of 16 value channels]
+// [key channel][16] (value channels rounded up to a multiple of 16; the channels beyond stay zero), so that the part
+// of a line that one workgroup of the walk owns is one run of memory. Two kernels: the
 // step before the walk (a short causal convolution with silu over the q, k and v columns of a 32-bit input product,
 // unit q and k per head, beta) and the walk itself. Everything is 32-bit.
 //
-// A request's state line holds S [heads][dim][vdim] and, from float `conv_at` on, the convolution's last taps - 1
+// A request's state line holds S and, from float `conv_at` on, the convolution's last taps - 1
 // inputs [taps - 1][channels], oldest first. Rows of the step are grouped by request: request s owns the rows
 // [cu_rows[s], cu_rows[s + 1]) in order of position and the line seq_slots[s].
 #include "common.h"
@@ -111,12 +113,10 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   const int hq = h / (H / G);
   constexpr int Dp = 16 * R;                 // key channels as the lanes hold them (those from D on are zeros)
   constexpr int stride = 3 * Dp + 20;
-  float* S_line = state + (long)seq_slots[s] * lds + (long)h * D * V;
-  // the line's [D][16 channels of this block] into LDS in runs of 16, then each lane's own elements
-  for (int e = t; e < D * 16; e += 256) {
-    const int d = e / 16, cc = vb * 16 + e % 16;
-    dr_lds[e] = cc < V ? S_line[(long)d * V + cc] : 0.f;
-  }
+  // this block's [D][16] part of the line: one run of memory, into LDS 16 bytes a lane, then each lane's own elements
+  float* S_line = state + (long)seq_slots[s] * lds + ((long)h * gridDim.x + vb) * D * 16;
+  for (int e = t; e < D * 4; e += 256)
+    reinterpret_cast<float4*>(dr_lds)[e] = reinterpret_cast<const float4*>(S_line)[e];
   __syncthreads();
   float S[R];
 #pragma unroll
@@ -219,10 +219,9 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     if (d < D) dr_lds[d * 16 + cl] = S[i];
   }
   __syncthreads();
-  for (int e = t; e < D * 16; e += 256) {
-    const int d = e / 16, cc = vb * 16 + e % 16;
-    if (cc < V) S_line[(long)d * V + cc] = dr_lds[e];
-  }
+  // (channels beyond vdim have seen values of zero only and are still zero)
+  for (int e = t; e < D * 4; e += 256)
+    reinterpret_cast<float4*>(S_line)[e] = reinterpret_cast<const float4*>(dr_lds)[e];
 }
 
 TIS_EXPORT int tis_delta_prepare(const float* proj, long ldp, int conv_off, int beta_off, const float* taps, int K,
@@ -244,8 +243,10 @@ TIS_EXPORT int tis_delta_scan(const float* u, long ldu, int q_off, int k_off, in
                               long ldd, float* state, long lds, const int* cu_rows, const int* seq_slots, int n_seqs,
                               float* out, long ldo, int H, int G, int D, int V, hipStream_t stream) {
   if (n_seqs == 0) return 0;
-  if (n_seqs < 0 || n_seqs > 65535 || H < 1 || H > 65535 || G < 1 || H % G || D < 1 || D > 256 || V < 1)
-    return tis_fail("delta_scan: bad size requests=%d heads=%d qk_heads=%d dim=%d (at most 256) vdim=%d", n_seqs, H, G, D, V);
+  if (n_seqs < 0 || n_seqs > 65535 || H < 1 || H > 65535 || G < 1 || H % G || D < 1 || D > 256 || V < 1 || lds % 4 ||
+      ((uintptr_t)state % 16))
+    return tis_fail("delta_scan: bad size requests=%d heads=%d qk_heads=%d dim=%d (at most 256) vdim=%d, or state lines that are "
+                    "not 16 bytes aligned", n_seqs, H, G, D, V);
   const int R = D <= 16 ? 1 : D <= 32 ? 2 : D <= 64 ? 4 : D <= 128 ? 8 : 16;
   const int tokens = R <= 8 ? 16 : 8;
   size_t lds_bytes = 2 * (size_t)tokens * (3 * 16 * R + 20) * sizeof(float);      // two buffers of rows

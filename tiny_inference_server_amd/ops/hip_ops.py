@@ -1947,12 +1947,15 @@ class HipOps:
         """Walk the step's rows of every request through its matrix state, in order: per head S <- diag(decay) S;
         w = beta (v - S^T k); S <- S + k w^T; o = S^T q. Returns o [rows, heads * vdim] 32-bit. u: [rows, ...] 32-bit with
         q and k (qk_heads * dim each; head h reads those of qk head h // (heads / qk_heads)), v (heads * vdim) and beta
-        (heads) at the given columns; decay [rows, heads * dim]; state: [slots, floats] 32-bit, S [heads, dim, vdim] first."""
+        (heads) at the given columns; decay [rows, heads * dim]; state: [slots, floats] 32-bit, a line starting with S as
+        [heads, blocks of 16 value channels, dim, 16] (lines 16 bytes aligned)."""
         n = u.shape[0]
         self._f32_rows(u, "delta_scan rows", n, max(q_off + qk_heads * dim, k_off + qk_heads * dim, v_off + n_heads * vdim,
                                                     beta_off + n_heads))
         self._f32_rows(decay, "delta_scan decays", n, n_heads * dim)
-        self._check_lines("delta_scan", state, n_heads * dim * vdim, batch)
+        self._check_lines("delta_scan", state, n_heads * -(-vdim // 16) * dim * 16, batch)
+        if state.stride(0) % 4 or state.data_ptr() % 16:
+            raise KernelError("delta_scan: state lines must be 16 bytes aligned")
         out = torch.empty(n, n_heads * vdim, dtype=torch.float32, device=self.device)
         self._lazy("delta_rule").tis_delta_scan(
             _ptr(u), u.stride(0), int(q_off), int(k_off), int(v_off), int(beta_off), _ptr(decay), decay.stride(0), _ptr(state),

@@ -243,6 +243,12 @@ class SelectiveStateSpace:
         return self.ops.linear(self.core(proj, ctx), self.w_o, residual=residual)
 
 
+def delta_state_floats(n_heads: int, dim: int, vdim: int) -> int:
+    """32-bit floats of a delta rule's matrix state in a request's line: [heads, blocks of 16 value channels, dim, 16],
+    the value channels rounded up to whole blocks (a block is what one workgroup of the walk owns: one run of memory)."""
+    return n_heads * -(-vdim // 16) * dim * 16
+
+
 @MIXERS.register("gated_delta_rule")
 class GatedDeltaRule:
     """A matrix state per head that is corrected towards each new value instead of only added to, with a decay per key
@@ -257,8 +263,8 @@ class GatedDeltaRule:
     Each head's o is divided by its root mean square over vdim (eps under the root), times a gain of vdim entries that
     the heads share, times sigmoid((x.Wg1^T).Wg2^T); then Wo. Everything between the convolution and the gate is 32-bit.
 
-    A request's state line holds S [heads, dim, vdim] and after it the convolution's last taps - 1 inputs
-    [taps - 1, channels]; a line that is taken anew is all zeros.
+    A request's state line holds S as [heads, blocks of 16 value channels, dim, 16] (`delta_state_floats`) and after it
+    the convolution's last taps - 1 inputs [taps - 1, channels]; a line that is taken anew is all zeros.
 
     params: width, n_heads, qk_heads, dim, vdim, taps, decay_rank, gate_rank, eps. tensors, stored [out, in]: q, k
     (qk_heads*dim, width), v (heads*vdim, width), q_conv, k_conv, v_conv ([channels, taps], the last column weighs the
@@ -283,7 +289,8 @@ class GatedDeltaRule:
     @classmethod
     def cache_need(cls, params):
         H, G, D, V, K, C = cls._sizes(params)
-        return StateNeed((H * D * V + (K - 1) * C,), "float32")
+        floats = delta_state_floats(H, D, V) + (K - 1) * C
+        return StateNeed((floats + -floats % 4,), "float32")        # (lines start 16 bytes aligned)
 
     def __init__(self, spec, tensors, ops):
         p = spec.params
@@ -307,7 +314,7 @@ class GatedDeltaRule:
         self.w_g2 = to_gain(ops, tensors.of(spec, "g2"))
         self.norm_gain = to_gain(ops, tensors.of(spec, "norm"))
         self.w_o = to_compute(ops, tensors.of(spec, "o"))
-        self.conv_at = self.H * self.D * self.V                                  # where the line's convolution inputs start
+        self.conv_at = delta_state_floats(self.H, self.D, self.V)                # where the line's convolution inputs start
 
     def core(self, proj, ctx):
         ops, b, at = self.ops, ctx.batch, self.at
